@@ -65,6 +65,7 @@ def build(force: bool = False, jobs: int = 8, verbose: bool = True) -> Path:
         want.append(obj)
         if force or _newer(src, obj, kernel_hdrs):
             cmd = [HIPCC, f"--offload-arch={ARCH}", *common, "-munsafe-fp-atomics",
+                   "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                    "-Wno-unused-result", "-c", str(src), "-o", str(obj)]
             jobs_list.append(cmd)
     host_flags = [

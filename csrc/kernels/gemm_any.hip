@@ -1,0 +1,268 @@
+// Row-major GEMM of any shape: out = epi(A W^T) with W stored [N][K] as checkpoints hold it.
+//
+// It serves what the fragment-packed GEMMs (gemm.hip, gemm_prefill.hip) do not take: fp32 models (true
+// fp32 FMA, no reduced-precision matrix mode), sizes that are not multiples of the MFMA tile, one
+// product per head (batch = blockIdx.z with strides on A, W and out), one product per expert over a
+// device-side row grouping (group_off; tiles are located on the device, so the grid is fixed and
+// the launch is graph-capturable), A-row gathers, and gated pairs (two weight matrices, one
+// activation in the epilogue).
+//   bf16: 64 x 64 block tile, 4 waves of 2 x 2 v_mfma_f32_16x16x32_bf16 tiles, operands read as 16-B
+//         fragments straight from global memory (both operands are k-contiguous rows), fp32 accumulate.
+//   fp32: 64 x 64 x 16 LDS-tiled FMA kernel, 4 x 4 outputs per thread, k ascending.
+#include <cstdlib>
+
+#include "common.h"
+#include "seq_launchers.h"
+
+namespace vgate {
+namespace {
+
+constexpr int BM = 64, BN = 64;
+
+__device__ __forceinline__ bool locate_tile(const AnyGemmArgs& p, int by, int& grp, int& r0, int& rend) {
+  if (p.group_off == nullptr) {
+    grp = 0; r0 = by * BM; rend = p.M;
+    return r0 < p.M;
+  }
+  int base = 0;
+  for (int g = 0; g < p.groups; ++g) {
+    const int a = p.group_off[g], b = p.group_off[g + 1];
+    const int nt = (b - a + BM - 1) / BM;
+    if (by < base + nt) {
+      grp = g; r0 = a + (by - base) * BM; rend = b;
+      return true;
+    }
+    base += nt;
+  }
+  return false;
+}
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
+
+__device__ __forceinline__ float epi_val(const AnyGemmArgs& p, float g, float u) {
+  if (p.act == 1) return g * sigmoidf_(g) * u;
+  if (p.act == 2) {
+    const float gg = fminf(g, p.limit);
+    const float uu = fminf(fmaxf(u, -p.limit), p.limit);
+    return gg * sigmoidf_(p.alpha * gg) * (uu + 1.f);
+  }
+  if (p.act == 3) return tanhf(g);
+  return g;
+}
+
+__device__ __forceinline__ void store_out(const AnyGemmArgs& p, int64_t b, int m, int n, float v) {
+  if (p.gate != nullptr) {
+    const int64_t gi = (int64_t)m * p.ldg + b * p.g_bs + n;
+    const float gl = p.gate_f32 ? reinterpret_cast<const float*>(p.gate)[gi]
+                                : bf2f(reinterpret_cast<const bf16_t*>(p.gate)[gi]);
+    v *= sigmoidf_(gl);
+  }
+  const int64_t oi = (int64_t)m * p.ldo + b * p.o_bs + n;
+  if (p.out_f32) reinterpret_cast<float*>(p.out)[oi] = v;
+  else reinterpret_cast<bf16_t*>(p.out)[oi] = f2bf(v);
+}
+
+__device__ __forceinline__ bf16x8 load_frag(const bf16_t* rowp, int k, int K, bool valid) {
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (valid && k < K) {
+    const bf16_t* q = rowp + k;
+    if (k + 8 <= K && (reinterpret_cast<uintptr_t>(q) & 15) == 0) {
+      v = ld16(q);
+    } else {
+      uint32_t w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = (k + 2 * j < K) ? q[2 * j] : 0;
+        const uint32_t hi = (k + 2 * j + 1 < K) ? q[2 * j + 1] : 0;
+        w[j] = lo | (hi << 16);
+      }
+      v = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  }
+  return as_bf16x8(v);
+}
+
+template <int DUAL>
+__global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
+  int grp, r0, rend;
+  if (!locate_tile(p, blockIdx.y, grp, r0, rend)) return;
+  const int64_t b = blockIdx.z;
+  const int64_t wsel = (p.group_off != nullptr) ? grp : b;
+  const int n0 = blockIdx.x * BN;
+  const int l = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int wm = wv & 1, wn = wv >> 1;
+  const int lr = l & 15, lk = 8 * (l >> 4);
+  const bf16_t* A = reinterpret_cast<const bf16_t*>(p.a) + b * p.a_bs;
+  const bf16_t* W = reinterpret_cast<const bf16_t*>(p.w) + wsel * p.w_bs;
+  const bf16_t* W2 = DUAL ? reinterpret_cast<const bf16_t*>(p.w2) + wsel * p.w_bs : nullptr;
+  const bf16_t* arow[2];
+  bool aval[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m = r0 + wm * 32 + i * 16 + lr;
+    aval[i] = m < rend;
+    const int src = aval[i] ? (p.a_rows ? p.a_rows[m] : m) : 0;
+    arow[i] = A + (int64_t)src * p.lda;
+  }
+  const bf16_t* wrow[2];
+  const bf16_t* w2row[2];
+  bool wval[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int n = n0 + wn * 32 + j * 16 + lr;
+    wval[j] = n < p.N;
+    wrow[j] = W + (int64_t)(wval[j] ? n : 0) * p.ldw;
+    w2row[j] = DUAL ? W2 + (int64_t)(wval[j] ? n : 0) * p.ldw : nullptr;
+  }
+  f32x4 acc[2][2], acc2[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      acc2[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  for (int k0 = 0; k0 < p.K; k0 += 32) {
+    const int k = k0 + lk;
+    bf16x8 af[2], bfr[2], b2[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) af[i] = load_frag(arow[i], k, p.K, aval[i]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      bfr[j] = load_frag(wrow[j], k, p.K, wval[j]);
+      if (DUAL) b2[j] = load_frag(w2row[j], k, p.K, wval[j]);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        acc[i][j] = mfma16(af[i], bfr[j], acc[i][j]);
+        if (DUAL) acc2[i][j] = mfma16(af[i], b2[j], acc2[i][j]);
+      }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wn * 32 + j * 16 + lr;
+      if (n >= p.N) continue;
+      const float bias = p.bias ? p.bias[n] : 0.f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int m = r0 + wm * 32 + i * 16 + 4 * (l >> 4) + e;
+        if (m >= rend) continue;
+        store_out(p, b, m, n, epi_val(p, acc[i][j][e] + bias, DUAL ? acc2[i][j][e] : 0.f));
+      }
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ float ldf(const T* q);
+template <>
+__device__ __forceinline__ float ldf<float>(const float* q) { return *q; }
+template <>
+__device__ __forceinline__ float ldf<bf16_t>(const bf16_t* q) { return bf2f(*q); }
+
+constexpr int BK = 16;
+
+template <typename T, int DUAL>
+__global__ __launch_bounds__(256) void gemm_any_fma_kernel(AnyGemmArgs p) {
+  __shared__ float As[BK][BM + 4];
+  __shared__ float Ws[BK][BN + 4];
+  __shared__ float Us[DUAL ? BK : 1][BN + 4];
+  int grp, r0, rend;
+  if (!locate_tile(p, blockIdx.y, grp, r0, rend)) return;
+  const int64_t b = blockIdx.z;
+  const int64_t wsel = (p.group_off != nullptr) ? grp : b;
+  const int n0 = blockIdx.x * BN;
+  const int tid = threadIdx.x;
+  const int tx = tid & 15, ty = tid >> 4;
+  const T* A = reinterpret_cast<const T*>(p.a) + b * p.a_bs;
+  const T* W = reinterpret_cast<const T*>(p.w) + wsel * p.w_bs;
+  const T* W2 = DUAL ? reinterpret_cast<const T*>(p.w2) + wsel * p.w_bs : nullptr;
+  // loader: row tid >> 2 of the tile, 4 consecutive k from (tid & 3) * 4
+  const int lrow = tid >> 2, lk = (tid & 3) * 4;
+  const int am = r0 + lrow;
+  const bool aok = am < rend;
+  const T* ap = A + (int64_t)(aok ? (p.a_rows ? p.a_rows[am] : am) : 0) * p.lda;
+  const int wn_ = n0 + lrow;
+  const bool wok = wn_ < p.N;
+  const T* wp = W + (int64_t)(wok ? wn_ : 0) * p.ldw;
+  const T* up = DUAL ? W2 + (int64_t)(wok ? wn_ : 0) * p.ldw : nullptr;
+  float acc[4][4], acc2[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { acc[i][j] = 0.f; acc2[i][j] = 0.f; }
+  for (int k0 = 0; k0 < p.K; k0 += BK) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int k = k0 + lk + e;
+      const bool kin = k < p.K;
+      As[lk + e][lrow] = (aok && kin) ? ldf<T>(ap + k) : 0.f;
+      Ws[lk + e][lrow] = (wok && kin) ? ldf<T>(wp + k) : 0.f;
+      if (DUAL) Us[lk + e][lrow] = (wok && kin) ? ldf<T>(up + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < BK; ++k) {
+      float av[4], wv[4], uv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = As[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        wv[j] = Ws[k][tx * 4 + j];
+        uv[j] = DUAL ? Us[k][tx * 4 + j] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+          if (DUAL) acc2[i][j] = fmaf(av[i], uv[j], acc2[i][j]);
+        }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = r0 + ty * 4 + i;
+    if (m >= rend) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n >= p.N) continue;
+      const float bias = p.bias ? p.bias[n] : 0.f;
+      store_out(p, b, m, n, epi_val(p, acc[i][j] + bias, DUAL ? acc2[i][j] : 0.f));
+    }
+  }
+}
+
+bool simple_only() {
+  static const bool v = [] {
+    const char* e = getenv("VGATE_GEMM_ANY_FMA");
+    return e != nullptr && e[0] == '1';
+  }();
+  return v;
+}
+
+}  // namespace
+
+void launch_gemm_any(const AnyGemmArgs& g, hipStream_t st) {
+  if (g.M <= 0 || g.N <= 0 || g.batch <= 0) return;
+  const int mt = (g.M + BM - 1) / BM + (g.group_off ? g.groups : 0);
+  const dim3 grid((g.N + BN - 1) / BN, mt, g.batch), block(256);
+  const bool dual = g.w2 != nullptr;
+  if (g.in_f32) {
+    if (dual) hipLaunchKernelGGL((gemm_any_fma_kernel<float, 1>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((gemm_any_fma_kernel<float, 0>), grid, block, 0, st, g);
+  } else if (simple_only()) {
+    if (dual) hipLaunchKernelGGL((gemm_any_fma_kernel<bf16_t, 1>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((gemm_any_fma_kernel<bf16_t, 0>), grid, block, 0, st, g);
+  } else {
+    if (dual) hipLaunchKernelGGL((gemm_any_mfma_kernel<1>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((gemm_any_mfma_kernel<0>), grid, block, 0, st, g);
+  }
+}
+
+}  // namespace vgate

@@ -1,0 +1,182 @@
+// Row-wise kernels of layered hybrid models over an fp32 residual stream: embedding gather into
+// fp32, RMS norm with a scalar or vector weight (fp32 statistics, bf16 or fp32 rows in and out,
+// optional row gather), the gated residual update of a parallel layer, and mixture-of-experts
+// routing (sigmoid scores with a selection-only correction, top-k, counting sort by expert, weighted
+// combine). Every kernel reads its sizes from arguments and its per-step metadata from device
+// memory, so the launches are graph-capturable.
+#include "common.h"
+#include "seq_launchers.h"
+
+namespace vgate {
+namespace {
+
+__device__ __forceinline__ float ldx(const void* p, int64_t i, int f32) {
+  return f32 ? reinterpret_cast<const float*>(p)[i] : bf2f(reinterpret_cast<const bf16_t*>(p)[i]);
+}
+__device__ __forceinline__ void stx(void* p, int64_t i, int f32, float v) {
+  if (f32) reinterpret_cast<float*>(p)[i] = v;
+  else reinterpret_cast<bf16_t*>(p)[i] = f2bf(v);
+}
+__device__ __forceinline__ float sigm(float x) { return 1.f / (1.f + expf(-x)); }
+
+__global__ __launch_bounds__(256) void norm_rows_kernel(const void* __restrict__ x, int64_t ldx_, int x_f32,
+                                                         const int32_t* __restrict__ rows,
+                                                         const float* __restrict__ w, int w_scalar, float eps,
+                                                         void* __restrict__ y, int64_t ldy, int y_f32, int n) {
+  __shared__ float red[16];
+  const int m = blockIdx.x;
+  const int64_t src = rows ? rows[m] : m;
+  const int64_t xo = src * ldx_;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < n; c += blockDim.x) {
+    const float v = ldx(x, xo + c, x_f32);
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_reduce_sum(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)n + eps);
+  const float ws = w_scalar ? w[0] : 1.f;
+  for (int c = threadIdx.x; c < n; c += blockDim.x) {
+    const float v = ldx(x, xo + c, x_f32) * inv * (w_scalar ? ws : w[c]);
+    stx(y, (int64_t)m * ldy + c, y_f32, v);
+  }
+}
+
+__global__ __launch_bounds__(256) void embed_rows_kernel(const int32_t* __restrict__ ids,
+                                                          const int32_t* __restrict__ prev,
+                                                          const void* __restrict__ table, int t_f32,
+                                                          float* __restrict__ x, int W, int vocab) {
+  const int t = blockIdx.x;
+  int tok = ids[t];
+  if (tok < 0 && prev != nullptr) tok = prev[-tok - 1];
+  const bool ok = tok >= 0 && tok < vocab;
+  for (int c = threadIdx.x; c < W; c += blockDim.x)
+    x[(int64_t)t * W + c] = ok ? ldx(table, (int64_t)tok * W + c, t_f32) : 0.f;
+}
+
+__global__ __launch_bounds__(256) void gated_residual_kernel(float* __restrict__ x, const void* __restrict__ y1,
+                                                              const void* __restrict__ g1, int64_t ldg1,
+                                                              const float* __restrict__ b1,
+                                                              const void* __restrict__ y2,
+                                                              const void* __restrict__ g2, int64_t ldg2,
+                                                              const float* __restrict__ b2, int f32, int W) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const int64_t i = (int64_t)t * W + c;
+    float v = ldx(y1, i, f32);
+    if (g1 != nullptr) v *= sigm(ldx(g1, (int64_t)t * ldg1 + c, f32) + (b1 ? b1[c] : 0.f));
+    if (y2 != nullptr) {
+      float u = ldx(y2, i, f32);
+      if (g2 != nullptr) u *= sigm(ldx(g2, (int64_t)t * ldg2 + c, f32) + (b2 ? b2[c] : 0.f));
+      v += u;
+    }
+    x[i] += v;
+  }
+}
+
+// one thread per token: `top` rounds of arg-max over the corrected scores (lowest index wins a tie)
+__global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ z, const float* __restrict__ corr,
+                                                        int T, int E, int top, float norm_eps,
+                                                        int32_t* __restrict__ idx, float* __restrict__ wts) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const float* zr = z + (int64_t)t * E;
+  float sum = 0.f;
+  for (int c = 0; c < top; ++c) {
+    int best = -1;
+    float bv = -INFINITY, bs = 0.f;
+    for (int e = 0; e < E; ++e) {
+      bool taken = false;
+      for (int d = 0; d < c; ++d) taken |= idx[(int64_t)t * top + d] == e;
+      if (taken) continue;
+      const float s = sigm(zr[e]);
+      const float v = s + (corr ? corr[e] : 0.f);
+      if (best < 0 || v > bv) { best = e; bv = v; bs = s; }
+    }
+    idx[(int64_t)t * top + c] = best;
+    wts[(int64_t)t * top + c] = bs;
+    sum += bs;
+  }
+  const float inv = 1.f / (sum + norm_eps);
+  for (int c = 0; c < top; ++c) wts[(int64_t)t * top + c] *= inv;
+}
+
+// single workgroup: histogram, exclusive scan, placement (token order inside a group is arbitrary:
+// every row of a grouped GEMM is computed independently of its neighbours)
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* __restrict__ idx, int n, int E,
+                                                         int top, int32_t* __restrict__ rows,
+                                                         int32_t* __restrict__ pos, int32_t* __restrict__ off) {
+  extern __shared__ int32_t cnt[];  // [E] counts, then [E] cursors
+  int32_t* cur = cnt + E;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&cnt[idx[i]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int a = 0;
+    for (int e = 0; e < E; ++e) {
+      off[e] = a; cur[e] = a;
+      a += cnt[e];
+    }
+    off[E] = a;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int p = atomicAdd(&cur[idx[i]], 1);
+    rows[p] = i / top;
+    pos[i] = p;
+  }
+}
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(const void* __restrict__ y, const int32_t* __restrict__ pos,
+                                                           const float* __restrict__ wts, int W, int top, int f32,
+                                                           void* __restrict__ out) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float a = 0.f;
+    for (int k = 0; k < top; ++k)
+      a = fmaf(wts[(int64_t)t * top + k], ldx(y, (int64_t)pos[(int64_t)t * top + k] * W + c, f32), a);
+    stx(out, (int64_t)t * W + c, f32, a);
+  }
+}
+
+}  // namespace
+
+void launch_norm_rows(const void* x, int64_t ldx_, int x_f32, const int32_t* rows, const float* w, int w_scalar,
+                      float eps, void* y, int64_t ldy, int y_f32, int M, int n, hipStream_t st) {
+  if (M <= 0) return;
+  hipLaunchKernelGGL(norm_rows_kernel, dim3(M), dim3(256), 0, st, x, ldx_, x_f32, rows, w, w_scalar, eps, y, ldy,
+                     y_f32, n);
+}
+
+void launch_embed_rows(const int32_t* ids, const int32_t* prev, const void* table, int t_f32, float* x, int T, int W,
+                       int vocab, hipStream_t st) {
+  if (T <= 0) return;
+  hipLaunchKernelGGL(embed_rows_kernel, dim3(T), dim3(256), 0, st, ids, prev, table, t_f32, x, W, vocab);
+}
+
+void launch_gated_residual(float* x, const void* y1, const void* g1, int64_t ldg1, const float* b1, const void* y2,
+                           const void* g2, int64_t ldg2, const float* b2, int f32, int T, int W, hipStream_t st) {
+  if (T <= 0) return;
+  hipLaunchKernelGGL(gated_residual_kernel, dim3(T), dim3(256), 0, st, x, y1, g1, ldg1, b1, y2, g2, ldg2, b2, f32, W);
+}
+
+void launch_moe_route(const float* z, const float* corr, int T, int E, int top, float norm_eps, int32_t* idx,
+                      float* wts, hipStream_t st) {
+  if (T <= 0) return;
+  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 63) / 64), dim3(64), 0, st, z, corr, T, E, top, norm_eps, idx, wts);
+}
+
+void launch_moe_sort(const int32_t* idx, int T, int E, int top, int32_t* rows, int32_t* pos, int32_t* off,
+                     hipStream_t st) {
+  if (T <= 0) return;
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 2 * E * sizeof(int32_t), st, idx, T * top, E, top, rows,
+                     pos, off);
+}
+
+void launch_moe_combine(const void* y, const int32_t* pos, const float* wts, int T, int W, int top, int f32,
+                        void* out, hipStream_t st) {
+  if (T <= 0) return;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, st, y, pos, wts, W, top, f32, out);
+}
+
+}  // namespace vgate

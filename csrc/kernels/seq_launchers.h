@@ -1,0 +1,84 @@
+// Host-side launcher declarations for the kernels of layered hybrid models: row-major GEMMs of any
+// shape (batched per head, grouped per expert, gated-linear-unit pairs), row norms with a scalar or a
+// vector weight over an fp32 residual stream, latent (compressed key/value) attention over a paged
+// cache, the generalized delta rule over per-sequence state slots, and mixture-of-experts routing.
+// Activations are bf16 or fp32 (`f32` flags); the residual stream, scores, norms and states are fp32.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vgate {
+
+// out[b][m][n] = epi(sum_k A[b][row(m)][k] * W[g][n][k]); A, W both bf16 or both fp32 (in_f32).
+struct AnyGemmArgs {
+  const void* a = nullptr; int64_t lda = 0, a_bs = 0;
+  const int32_t* a_rows = nullptr;      // optional gather of A rows (device)
+  const void* w = nullptr; const void* w2 = nullptr;  // w2: the "up" matrix of a gated pair (same layout)
+  int64_t ldw = 0, w_bs = 0;            // w_bs: stride between batches / groups
+  const float* bias = nullptr;          // [N] added to the accumulator (single-matrix form)
+  const void* gate = nullptr; int64_t ldg = 0, g_bs = 0;  // out *= sigmoid(gate[m][n]) (activation dtype)
+  void* out = nullptr; int64_t ldo = 0, o_bs = 0;
+  int M = 0, N = 0, K = 0, batch = 1;
+  const int32_t* group_off = nullptr;   // [groups + 1] row ranges (device): rows of group g use W + g * w_bs
+  int groups = 0;
+  int act = 0;                          // 0 none; 1 silu(g) * u; 2 clamped: g' = min(g, L), u' = clamp(u, -L, L),
+  float limit = 0.f;                    //   g' * sigmoid(alpha g') * (u' + 1); 3 tanh (single matrix)
+  float alpha = 1.702f;
+  int in_f32 = 0, out_f32 = 0, gate_f32 = 0;
+};
+void launch_gemm_any(const AnyGemmArgs& g, hipStream_t st);
+
+// y[m][:] = x[row(m)][:] * rsqrt(mean(x^2) + eps) * w   (w: one number if w_scalar, else [n])
+void launch_norm_rows(const void* x, int64_t ldx, int x_f32, const int32_t* rows, const float* w, int w_scalar,
+                      float eps, void* y, int64_t ldy, int y_f32, int M, int n, hipStream_t st);
+// x[t][:] = table[id(t)][:] as fp32; ids < 0 name the previous step's sample prev[-id - 1]
+void launch_embed_rows(const int32_t* ids, const int32_t* prev, const void* table, int t_f32, float* x, int T, int W,
+                       int vocab, hipStream_t st);
+// x += y1 * sigmoid(g1 + b1) [+ y2 * sigmoid(g2 + b2)]; null g: plain add
+void launch_gated_residual(float* x, const void* y1, const void* g1, int64_t ldg1, const float* b1, const void* y2,
+                           const void* g2, int64_t ldg2, const float* b2, int f32, int T, int W, hipStream_t st);
+
+struct LatentArgs {
+  int rank = 0, rot = 0, rot_dims = 0;  // latent size, rotated key size, leading rotated dims (<= rot, even)
+  const float* inv_freq = nullptr;      // [rot_dims / 2]
+  const int32_t* positions = nullptr;   // [T]
+  const int32_t* slots = nullptr;       // [T] cache row of each token (-1: padding)
+  void* cache = nullptr;                // [pages * page][rank + rot]
+  int f32 = 0;
+  int T = 0;
+};
+// cache[slot] = [rmsnorm(kv[:rank]) * w, rope(kv[rank:])]
+void launch_latent_write(const LatentArgs& a, const void* kv, int64_t ldkv, const float* w, float eps, hipStream_t st);
+// qa[t][h][rank:] = rope(q[t][h][dim:]) for q laid out [T][H][dim + rot], qa [T][H][rank + rot]
+void launch_latent_qrope(const LatentArgs& a, const void* q, int H, int dim, void* qa, hipStream_t st);
+// ol[t][h][:rank] = softmax_j(scale * qa[t][h] . cache[j]) . cache[j][:rank] over the causal keys
+void launch_latent_attn(const LatentArgs& a, const void* qa, int H, float scale, const int32_t* block_tables,
+                        int max_blocks, int page, const int32_t* context_lens, const int32_t* query_start, int S,
+                        void* ol, hipStream_t st);
+
+struct DeltaArgs {
+  const void* r = nullptr; const void* k = nullptr; const void* v = nullptr; const void* g = nullptr;
+  const void* a = nullptr; int64_t ld = 0;      // rows of the fused projection (activation dtype), one stride
+  const void* wl = nullptr; int64_t ldw = 0;    // decay pre-activation rows
+  const float* w0 = nullptr; const float* ab = nullptr; const float* nw = nullptr;  // [H * D]
+  float decay_c = 0.f, unit_eps = 0.f, eps = 0.f;
+  float* state = nullptr;                       // [slots][H][D][D] (key-major)
+  const int32_t* state_slots = nullptr;         // [S] (-1: padding)
+  const int32_t* context_lens = nullptr; const int32_t* query_start = nullptr;
+  void* out = nullptr; int64_t ldo = 0;
+  int S = 0, H = 0, D = 0, f32 = 0;
+};
+void launch_delta_rule(const DeltaArgs& a, hipStream_t st);
+
+// idx, wts [T][top]: the `top` largest of sigmoid(z) + corr; wts = sigmoid(z) of the chosen / their sum
+void launch_moe_route(const float* z, const float* corr, int T, int E, int top, float norm_eps, int32_t* idx,
+                      float* wts, hipStream_t st);
+// counting sort of the T * top (token, choice) pairs by expert: rows[p] = token, pos[t * top + c] = p,
+// off[E + 1] = group boundaries
+void launch_moe_sort(const int32_t* idx, int T, int E, int top, int32_t* rows, int32_t* pos, int32_t* off,
+                     hipStream_t st);
+// out[t] = sum_c wts[t][c] * y[pos[t][c]]
+void launch_moe_combine(const void* y, const int32_t* pos, const float* wts, int T, int W, int top, int f32,
+                        void* out, hipStream_t st);
+
+}  // namespace vgate

@@ -616,9 +616,12 @@ void custom_allgather(const Tensor& inp, Tensor& out, const std::vector<int64_t>
 
 }  // namespace
 
+void bind_seq(pybind11::module& m);  // csrc/runtime/bindings_seq.cpp: hybrid-model kernels
+
 PYBIND11_MODULE(_C, m) {
   m.doc() = "vgate gfx950 (MI355X) HIP kernels and native runtime";
   namespace py = pybind11;
+  bind_seq(m);
   m.def("gemm", &gemm, "fragment-packed MFMA GEMM (+RMSNorm prologue, split-K, fused epilogues; bf16 or AWQ int4)",
         py::arg("x"), py::arg("wp"), py::arg("N"), py::arg("K"), py::arg("out"), py::arg("epi") = 0,
         py::arg("bias") = py::none(), py::arg("res") = py::none(), py::arg("norm_w") = py::none(),

@@ -1,0 +1,297 @@
+// Torch bindings of the hybrid-model kernels (csrc/kernels/seq_launchers.h): shapes, dtypes and strides
+// are checked here, on the host, before anything is launched; every op runs on torch's current HIP
+// stream and allocates nothing, so a forward pass built from them is graph-capturable.
+#include <torch/extension.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/core/DeviceGuard.h>
+
+#include "../kernels/seq_launchers.h"
+
+namespace {
+
+using torch::Tensor;
+using OptT = c10::optional<Tensor>;
+
+hipStream_t cur_stream() { return at::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
+
+bool has(const OptT& t) { return t.has_value() && t->defined(); }
+
+int act_f32(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda(), name, " must be a GPU tensor");
+  TORCH_CHECK(t.scalar_type() == torch::kFloat32 || t.scalar_type() == torch::kBFloat16, name, ": bf16 or fp32");
+  TORCH_CHECK(t.dim() == 0 || t.stride(-1) == 1, name, " must be contiguous in its last dim");
+  return t.scalar_type() == torch::kFloat32 ? 1 : 0;
+}
+
+const float* f32p(const OptT& t, const char* name, int64_t n = -1) {
+  if (!has(t)) return nullptr;
+  TORCH_CHECK(t->is_cuda() && t->scalar_type() == torch::kFloat32 && t->is_contiguous(), name, ": contiguous fp32 GPU tensor");
+  if (n >= 0) TORCH_CHECK(t->numel() == n, name, " has ", t->numel(), " elements, expected ", n);
+  return t->data_ptr<float>();
+}
+
+const int32_t* i32p(const Tensor& t, const char* name, int64_t min_n) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kInt32 && t.is_contiguous(), name, ": contiguous int32 GPU tensor");
+  TORCH_CHECK(t.numel() >= min_n, name, " has ", t.numel(), " elements, needs ", min_n);
+  return t.data_ptr<int32_t>();
+}
+
+// a [M, K] or [B, M, K]; w (and w2) [N, K] or [B | G, N, K]; out [M, N] or [B, M, N]
+void gemm_any(const Tensor& a, const Tensor& w, Tensor& out, const OptT& w2, const OptT& bias, const OptT& gate,
+              const OptT& a_rows, const OptT& group_off, int64_t act, double limit, double alpha) {
+  vgate::AnyGemmArgs g;
+  g.in_f32 = act_f32(a, "a");
+  TORCH_CHECK(act_f32(w, "w") == g.in_f32, "gemm_any: a and w must share a dtype");
+  g.out_f32 = act_f32(out, "out");
+  const bool b3 = a.dim() == 3;
+  TORCH_CHECK((a.dim() == 2 || b3) && out.dim() == a.dim(), "gemm_any: a / out 2-D or 3-D");
+  const bool grouped = has(group_off);
+  const int64_t B = b3 ? a.size(0) : 1;
+  g.batch = (int)B;
+  g.M = (int)out.size(-2); g.N = (int)out.size(-1); g.K = (int)a.size(-1);
+  g.a = a.data_ptr(); g.lda = a.stride(-2); g.a_bs = b3 ? a.stride(0) : 0;
+  g.out = out.data_ptr(); g.ldo = out.stride(-2); g.o_bs = b3 ? out.stride(0) : 0;
+  if (b3) TORCH_CHECK(out.size(0) == B, "gemm_any: batch of out");
+  TORCH_CHECK(w.size(-1) == g.K && w.size(-2) == g.N, "gemm_any: w must be [.., N=", g.N, ", K=", g.K, "]");
+  TORCH_CHECK(g.lda >= g.K && g.ldo >= g.N, "gemm_any: row strides");
+  g.w = w.data_ptr(); g.ldw = w.stride(-2);
+  if (w.dim() == 3) {
+    g.w_bs = w.stride(0);
+    TORCH_CHECK(grouped || w.size(0) == B, "gemm_any: batch of w");
+  } else {
+    TORCH_CHECK(w.dim() == 2 && !grouped, "gemm_any: w 2-D (3-D when batched / grouped)");
+    g.w_bs = 0;
+  }
+  if (has(w2)) {
+    TORCH_CHECK(act_f32(*w2, "w2") == g.in_f32 && w2->sizes() == w.sizes() && w2->strides() == w.strides(),
+                "gemm_any: w2 must match w");
+    g.w2 = w2->data_ptr();
+    TORCH_CHECK(act == 1 || act == 2, "gemm_any: a weight pair needs act 1 or 2");
+  } else {
+    TORCH_CHECK(act == 0 || act == 3, "gemm_any: act 1 / 2 need a weight pair");
+  }
+  g.bias = f32p(bias, "bias", g.N);
+  TORCH_CHECK(!(g.bias && B > 1), "gemm_any: bias only without batch");
+  if (has(gate)) {
+    g.gate_f32 = act_f32(*gate, "gate");
+    TORCH_CHECK(gate->dim() == out.dim() && gate->size(-1) == g.N && gate->size(-2) >= g.M, "gemm_any: gate shape");
+    g.gate = gate->data_ptr(); g.ldg = gate->stride(-2); g.g_bs = b3 ? gate->stride(0) : 0;
+  }
+  const int64_t rows_in = a.size(-2);
+  if (has(a_rows)) {
+    g.a_rows = i32p(*a_rows, "a_rows", g.M);  // values < rows of a: produced by moe_sort from token ids
+  } else {
+    TORCH_CHECK(rows_in >= g.M, "gemm_any: a has ", rows_in, " rows < M=", g.M);
+  }
+  if (grouped) {
+    TORCH_CHECK(!b3 && w.dim() == 3, "gemm_any: grouped form takes 2-D a / out and 3-D w");
+    g.groups = (int)w.size(0);
+    g.group_off = i32p(*group_off, "group_off", g.groups + 1);
+  }
+  g.act = (int)act; g.limit = (float)limit; g.alpha = (float)alpha;
+  TORCH_CHECK(B <= 65535, "gemm_any: batch too large");
+  c10::DeviceGuard guard(a.device());
+  vgate::launch_gemm_any(g, cur_stream());
+}
+
+void norm_rows(const Tensor& x, const Tensor& w, double eps, Tensor& y, const OptT& rows, bool scalar) {
+  const int xf = act_f32(x, "x"), yf = act_f32(y, "y");
+  TORCH_CHECK(x.dim() == 2 && y.dim() == 2 && x.size(1) == y.size(1), "norm_rows: [M, n] rows");
+  const int64_t n = x.size(1), M = y.size(0);
+  const float* wp = f32p(w, "w", scalar ? 1 : n);
+  const int32_t* rp = nullptr;
+  if (has(rows)) rp = i32p(*rows, "rows", M);
+  else TORCH_CHECK(x.size(0) >= M, "norm_rows: x rows");
+  c10::DeviceGuard guard(x.device());
+  vgate::launch_norm_rows(x.data_ptr(), x.stride(0), xf, rp, wp, scalar ? 1 : 0, (float)eps, y.data_ptr(), y.stride(0),
+                          yf, (int)M, (int)n, cur_stream());
+}
+
+void embed_rows(const Tensor& ids, const Tensor& table, Tensor& x, const OptT& prev) {
+  const int tf = act_f32(table, "table");
+  TORCH_CHECK(table.dim() == 2 && table.is_contiguous(), "embed_rows: table [vocab, W]");
+  TORCH_CHECK(x.is_cuda() && x.scalar_type() == torch::kFloat32 && x.is_contiguous() && x.dim() == 2 &&
+              x.size(1) == table.size(1), "embed_rows: x fp32 [T, W]");
+  const int T = (int)x.size(0);
+  const int32_t* ip = i32p(ids, "ids", T);
+  const int32_t* pp = has(prev) ? i32p(*prev, "prev", 1) : nullptr;
+  c10::DeviceGuard guard(x.device());
+  vgate::launch_embed_rows(ip, pp, table.data_ptr(), tf, x.data_ptr<float>(), T, (int)x.size(1), (int)table.size(0),
+                           cur_stream());
+}
+
+void gated_residual(Tensor& x, const Tensor& y1, const OptT& g1, const OptT& b1, const OptT& y2, const OptT& g2,
+                    const OptT& b2) {
+  TORCH_CHECK(x.is_cuda() && x.scalar_type() == torch::kFloat32 && x.is_contiguous() && x.dim() == 2,
+              "gated_residual: x fp32 [T, W]");
+  const int T = (int)x.size(0), W = (int)x.size(1);
+  const int f = act_f32(y1, "y1");
+  auto chk = [&](const Tensor& t, const char* name, bool dense) {
+    TORCH_CHECK(act_f32(t, name) == f && t.dim() == 2 && t.size(0) >= T && t.size(1) == W, name, ": [T, W] of y1's dtype");
+    if (dense) TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+  };
+  chk(y1, "y1", true);
+  if (has(y2)) chk(*y2, "y2", true);
+  if (has(g1)) chk(*g1, "g1", false);
+  if (has(g2)) chk(*g2, "g2", false);
+  TORCH_CHECK(!has(g2) || has(y2), "gated_residual: g2 without y2");
+  c10::DeviceGuard guard(x.device());
+  vgate::launch_gated_residual(x.data_ptr<float>(), y1.data_ptr(), has(g1) ? g1->data_ptr() : nullptr,
+                               has(g1) ? g1->stride(0) : 0, f32p(b1, "b1", W), has(y2) ? y2->data_ptr() : nullptr,
+                               has(g2) ? g2->data_ptr() : nullptr, has(g2) ? g2->stride(0) : 0, f32p(b2, "b2", W), f,
+                               T, W, cur_stream());
+}
+
+vgate::LatentArgs latent_common(const Tensor& positions, const Tensor& inv_freq, int64_t rot_dims, int64_t rank,
+                                int64_t rot, int64_t T) {
+  vgate::LatentArgs a;
+  a.rank = (int)rank; a.rot = (int)rot; a.rot_dims = (int)rot_dims; a.T = (int)T;
+  TORCH_CHECK(rank > 0 && rot >= 0 && rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0, "latent: rank / rot sizes");
+  OptT f(inv_freq);
+  a.inv_freq = f32p(f, "inv_freq", rot_dims / 2);
+  a.positions = i32p(positions, "positions", T);
+  return a;
+}
+
+void latent_write(const Tensor& kv, const Tensor& w, double eps, const Tensor& positions, const Tensor& slots,
+                  const Tensor& inv_freq, int64_t rot_dims, Tensor& cache, int64_t rank) {
+  const int f = act_f32(kv, "kv");
+  TORCH_CHECK(kv.dim() == 2 && cache.dim() == 3 && cache.is_contiguous() && act_f32(cache, "cache") == f,
+              "latent_write: kv [T, rank + rot], cache [pages, page, rank + rot] of one dtype");
+  const int64_t rot = kv.size(1) - rank;
+  TORCH_CHECK(cache.size(2) == kv.size(1), "latent_write: cache row width");
+  auto a = latent_common(positions, inv_freq, rot_dims, rank, rot, kv.size(0));
+  a.slots = i32p(slots, "slots", kv.size(0));  // values < pages * page: written by the step's block tables
+  a.cache = cache.data_ptr(); a.f32 = f;
+  OptT wo(w);
+  c10::DeviceGuard guard(kv.device());
+  vgate::launch_latent_write(a, kv.data_ptr(), kv.stride(0), f32p(wo, "w", rank), (float)eps, cur_stream());
+}
+
+void latent_qrope(const Tensor& q, const Tensor& positions, const Tensor& inv_freq, int64_t rot_dims, Tensor& qa,
+                  int64_t H, int64_t dim, int64_t rank, int64_t rot) {
+  const int f = act_f32(q, "q");
+  TORCH_CHECK(q.dim() == 2 && q.is_contiguous() && q.size(1) == H * (dim + rot), "latent_qrope: q [T, H * (dim + rot)]");
+  TORCH_CHECK(act_f32(qa, "qa") == f && qa.is_contiguous() && qa.numel() == q.size(0) * H * (rank + rot),
+              "latent_qrope: qa [T, H, rank + rot]");
+  auto a = latent_common(positions, inv_freq, rot_dims, rank, rot, q.size(0));
+  a.f32 = f;
+  c10::DeviceGuard guard(q.device());
+  vgate::launch_latent_qrope(a, q.data_ptr(), (int)H, (int)dim, qa.data_ptr(), cur_stream());
+}
+
+void latent_attn(const Tensor& qa, const Tensor& cache, const Tensor& block_tables, const Tensor& context_lens,
+                 const Tensor& query_start, Tensor& ol, double scale, int64_t H, int64_t rank, int64_t rot) {
+  const int f = act_f32(qa, "qa");
+  const int64_t E = rank + rot;
+  TORCH_CHECK(qa.is_contiguous() && qa.numel() % (H * E) == 0, "latent_attn: qa [T, H, rank + rot]");
+  const int64_t T = qa.numel() / (H * E);
+  TORCH_CHECK(act_f32(ol, "ol") == f && ol.is_contiguous() && ol.numel() == T * H * rank, "latent_attn: ol [T, H, rank]");
+  TORCH_CHECK(cache.dim() == 3 && cache.is_contiguous() && act_f32(cache, "cache") == f && cache.size(2) == E,
+              "latent_attn: cache [pages, page, rank + rot]");
+  TORCH_CHECK(rank <= 4096 && 17 * (E + 1) * 4 <= 56 * 1024, "latent_attn: latent size out of range");
+  TORCH_CHECK(block_tables.dim() == 2, "latent_attn: block_tables [S, max_blocks]");
+  const int64_t S = block_tables.size(0);
+  vgate::LatentArgs a;
+  a.rank = (int)rank; a.rot = (int)rot; a.T = (int)T; a.f32 = f; a.cache = cache.data_ptr();
+  const int32_t* bt = i32p(block_tables, "block_tables", 1);
+  const int32_t* cl = i32p(context_lens, "context_lens", S);
+  const int32_t* qs = i32p(query_start, "query_start", S + 1);
+  c10::DeviceGuard guard(qa.device());
+  vgate::launch_latent_attn(a, qa.data_ptr(), (int)H, (float)scale, bt, (int)block_tables.size(1), (int)cache.size(1),
+                            cl, qs, (int)S, ol.data_ptr(), cur_stream());
+}
+
+void delta_rule(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor& g, const Tensor& a, const Tensor& wl,
+                const Tensor& w0, const Tensor& ab, const Tensor& nw, Tensor& state, const Tensor& state_slots,
+                const Tensor& context_lens, const Tensor& query_start, Tensor& out, double decay_c, double unit_eps,
+                double eps) {
+  vgate::DeltaArgs p;
+  p.f32 = act_f32(r, "r");
+  TORCH_CHECK(state.is_cuda() && state.scalar_type() == torch::kFloat32 && state.is_contiguous() && state.dim() == 4 &&
+              state.size(2) == state.size(3), "delta_rule: state fp32 [slots, H, D, D]");
+  p.H = (int)state.size(1); p.D = (int)state.size(2);
+  TORCH_CHECK(p.D >= 1 && p.D <= 128, "delta_rule: head size 1..128");
+  const int64_t HD = (int64_t)p.H * p.D;
+  const int64_t T = r.size(0);
+  for (const Tensor* t : {&r, &k, &v, &g, &a, &wl}) {
+    TORCH_CHECK(act_f32(*t, "delta_rule input") == p.f32 && t->dim() == 2 && t->size(0) == T && t->size(1) == HD,
+                "delta_rule: inputs [T, H * D] of one dtype");
+  }
+  for (const Tensor* t : {&k, &v, &g, &a}) TORCH_CHECK(t->stride(0) == r.stride(0), "delta_rule: one row stride");
+  TORCH_CHECK(act_f32(out, "out") == p.f32 && out.dim() == 2 && out.size(0) == T && out.size(1) == HD, "delta_rule: out");
+  p.r = r.data_ptr(); p.k = k.data_ptr(); p.v = v.data_ptr(); p.g = g.data_ptr(); p.a = a.data_ptr(); p.ld = r.stride(0);
+  p.wl = wl.data_ptr(); p.ldw = wl.stride(0);
+  OptT o0(w0), o1(ab), o2(nw);
+  p.w0 = f32p(o0, "w0", HD); p.ab = f32p(o1, "ab", HD); p.nw = f32p(o2, "nw", HD);
+  p.decay_c = (float)decay_c; p.unit_eps = (float)unit_eps; p.eps = (float)eps;
+  p.state = state.data_ptr<float>();
+  p.S = (int)state_slots.numel();
+  p.state_slots = i32p(state_slots, "state_slots", p.S);  // values < slots (or -1): set by the slot manager
+  p.context_lens = i32p(context_lens, "context_lens", p.S);
+  p.query_start = i32p(query_start, "query_start", p.S + 1);  // values <= T: set by the step metadata
+  p.out = out.data_ptr(); p.ldo = out.stride(0);
+  c10::DeviceGuard guard(r.device());
+  vgate::launch_delta_rule(p, cur_stream());
+}
+
+void moe_route(const Tensor& z, const OptT& corr, int64_t top, double norm_eps, Tensor& idx, Tensor& wts) {
+  TORCH_CHECK(z.is_cuda() && z.scalar_type() == torch::kFloat32 && z.is_contiguous() && z.dim() == 2, "moe_route: z fp32 [T, E]");
+  const int64_t T = z.size(0), E = z.size(1);
+  TORCH_CHECK(top >= 1 && top <= E, "moe_route: top");
+  TORCH_CHECK(idx.is_cuda() && idx.scalar_type() == torch::kInt32 && idx.is_contiguous() && idx.numel() == T * top, "moe_route: idx");
+  TORCH_CHECK(wts.is_cuda() && wts.scalar_type() == torch::kFloat32 && wts.is_contiguous() && wts.numel() == T * top, "moe_route: wts");
+  c10::DeviceGuard guard(z.device());
+  vgate::launch_moe_route(z.data_ptr<float>(), f32p(corr, "corr", E), (int)T, (int)E, (int)top, (float)norm_eps,
+                          idx.data_ptr<int32_t>(), wts.data_ptr<float>(), cur_stream());
+}
+
+void moe_sort(const Tensor& idx, int64_t E, Tensor& rows, Tensor& pos, Tensor& off) {
+  TORCH_CHECK(idx.dim() == 2, "moe_sort: idx [T, top]");
+  const int64_t T = idx.size(0), top = idx.size(1);
+  TORCH_CHECK(E >= 1 && E <= 4096, "moe_sort: experts 1..4096");
+  const int32_t* ip = i32p(idx, "idx", T * top);
+  TORCH_CHECK(rows.numel() == T * top && pos.numel() == T * top && off.numel() == E + 1, "moe_sort: outputs");
+  i32p(rows, "rows", 0); i32p(pos, "pos", 0); i32p(off, "off", 0);
+  c10::DeviceGuard guard(idx.device());
+  vgate::launch_moe_sort(ip, (int)T, (int)E, (int)top, rows.data_ptr<int32_t>(), pos.data_ptr<int32_t>(),
+                         off.data_ptr<int32_t>(), cur_stream());
+}
+
+void moe_combine(const Tensor& y, const Tensor& pos, const Tensor& wts, Tensor& out) {
+  const int f = act_f32(y, "y");
+  TORCH_CHECK(out.dim() == 2 && out.is_contiguous() && act_f32(out, "out") == f && y.is_contiguous() && y.dim() == 2 &&
+              y.size(1) == out.size(1), "moe_combine: y [T * top, W], out [T, W]");
+  const int64_t T = out.size(0), W = out.size(1);
+  TORCH_CHECK(T > 0 && y.size(0) % T == 0, "moe_combine: rows of y");
+  const int64_t top = y.size(0) / T;
+  const int32_t* pp = i32p(pos, "pos", T * top);
+  OptT wo(wts);
+  c10::DeviceGuard guard(y.device());
+  vgate::launch_moe_combine(y.data_ptr(), pp, f32p(wo, "wts", T * top), (int)T, (int)W, (int)top, f, out.data_ptr(),
+                            cur_stream());
+}
+
+}  // namespace
+
+void bind_seq(pybind11::module& m) {
+  namespace py = pybind11;
+  m.def("gemm_any", &gemm_any, "row-major GEMM of any shape (batched / grouped / gated pair), bf16 MFMA or fp32 FMA",
+        py::arg("a"), py::arg("w"), py::arg("out"), py::arg("w2") = py::none(), py::arg("bias") = py::none(),
+        py::arg("gate") = py::none(), py::arg("a_rows") = py::none(), py::arg("group_off") = py::none(),
+        py::arg("act") = 0, py::arg("limit") = 0.0, py::arg("alpha") = 1.702);
+  m.def("norm_rows", &norm_rows, "RMS norm of rows, scalar or vector weight, fp32 statistics", py::arg("x"), py::arg("w"),
+        py::arg("eps"), py::arg("y"), py::arg("rows") = py::none(), py::arg("scalar") = false);
+  m.def("embed_rows", &embed_rows, "embedding gather into the fp32 residual stream", py::arg("ids"), py::arg("table"),
+        py::arg("x"), py::arg("prev") = py::none());
+  m.def("gated_residual", &gated_residual, "x += y1 * sigmoid(g1 + b1) + y2 * sigmoid(g2 + b2)", py::arg("x"),
+        py::arg("y1"), py::arg("g1") = py::none(), py::arg("b1") = py::none(), py::arg("y2") = py::none(),
+        py::arg("g2") = py::none(), py::arg("b2") = py::none());
+  m.def("latent_write", &latent_write, "latent norm + shared-key rotation + paged cache store");
+  m.def("latent_qrope", &latent_qrope, "rotate the rotated query part into the absorbed query buffer");
+  m.def("latent_attn", &latent_attn, "causal attention over the paged latent cache (absorbed projections)");
+  m.def("delta_rule", &delta_rule, "generalized delta rule recurrence over state slots + head norm + gate");
+  m.def("moe_route", &moe_route, "sigmoid router: corrected top-k choice, normalised uncorrected weights");
+  m.def("moe_sort", &moe_sort, "counting sort of (token, choice) pairs by expert");
+  m.def("moe_combine", &moe_combine, "weighted sum of a token's expert rows");
+}

@@ -118,21 +118,119 @@ def _from_hf_config(cfg: dict, name: str) -> ModelArch:
         bos_token_id=cfg.get("bos_token_id", 1) or 1, eos_token_ids=eos)
 
 
-def resolve_arch(model_id: str, overrides: dict | None = None) -> ModelArch:
+@dataclass(frozen=True)
+class LayerSpec:
+    """One layer of a layered hybrid model: which mixer it has (a key of
+    ``vgate.models.mixers.MIXERS``), the mixer's sizes and constants, its feed-forward (``None``:
+    the layer has none) and, for a layer without tensors of its own, the layer whose weights it
+    runs with (its cache or state stays its own)."""
+    kind: str
+    mixer: dict = field(hash=False, compare=False)
+    mlp: dict | None = field(default=None, hash=False, compare=False)
+    weights_of: int | None = None
+
+
+@dataclass(frozen=True)
+class HybridArch:
+    """A decoder made of a list of :class:`LayerSpec` over an fp32 residual stream."""
+    name: str
+    family: str
+    hidden_size: int
+    vocab_size: int
+    layers: tuple
+    rms_eps: float = 1e-6
+    max_position: int = 1 << 20
+    bos_token_id: int = 1
+    eos_token_ids: tuple = (2,)
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def owner(self, i: int) -> int:
+        """Index of the layer whose tensors layer ``i`` runs with."""
+        w = self.layers[i].weights_of
+        return i if w is None else int(w)
+
+    def num_params(self) -> int:
+        from vgate.models.mixers import layer_params
+        W = self.hidden_size
+        own = {self.owner(i) for i in range(len(self.layers))}
+        return 2 * self.vocab_size * W + 1 + sum(layer_params(self.layers[i], W) for i in sorted(own))
+
+    def to_dict(self) -> dict:
+        return asdict(self)
+
+
+def _zadirax_from_config(cfg: dict, name: str) -> HybridArch:
+    """config.json of the Zadirax design: every size and every constant that may differ between
+    models of the design is read here; nothing is inferred from a particular checkpoint."""
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        wo = L.get("weights_of")
+        if wo is not None and not (0 <= int(wo) < len(cfg["layers"])) or wo == i:
+            raise ValueError(f"layer {i}: weights_of {wo} names no other layer")
+        layers.append(LayerSpec(kind=L["type"], mixer=dict(L["mixer"]), mlp=dict(L["mlp"]) if L.get("mlp") else None,
+                                weights_of=None if wo is None else int(wo)))
+    for i, L in enumerate(layers):
+        if L.weights_of is not None and layers[L.weights_of].weights_of is not None:
+            raise ValueError(f"layer {i}: weights_of must name a layer that owns its tensors")
+    eos = cfg.get("eos_token_id", 2)
+    return HybridArch(name=name, family="zadirax", hidden_size=int(cfg["width"]), vocab_size=int(cfg["vocab"]),
+                      layers=tuple(layers), rms_eps=float(cfg["norm"]["eps"]),
+                      bos_token_id=int(cfg.get("bos_token_id", 1)),
+                      eos_token_ids=tuple(eos) if isinstance(eos, list) else (int(eos),))
+
+
+# config.json "architecture" -> parser of a layered hybrid design
+HYBRID_ARCHITECTURES = {"Zadirax": _zadirax_from_config}
+
+
+def _zadirax_preset(name: str, width: int, vocab: int, pairs: int, heads: int, dim: int, ff: int, experts: int,
+                    top: int, expert_ff: int, kv_rank: int, q_rank: int, rot: int, share: bool = False) -> HybridArch:
+    """Random-init Zadirax models (benchmarks, tests): ``pairs`` x [general_delta + dense, latent_attention + MoE]."""
+    delta = dict(kind="general_delta", mixer={"heads": heads, "dim": dim}, mlp={"kind": "dense", "ff": ff})
+    lat = dict(kind="latent_attention",
+               mixer={"heads": heads, "dim": dim, "rot_dim": rot, "vdim": dim, "kv_rank": kv_rank, "q_rank": q_rank,
+                      "rot": {"base": 10000.0, "dims": rot}, "scale": (dim + rot) ** -0.5},
+               mlp={"kind": "moe", "expert": {"ff": expert_ff, "limit": 7.0}, "router": {"experts": experts, "top": top}})
+    layers = []
+    for i in range(pairs):
+        layers.append(LayerSpec(**delta))
+        layers.append(LayerSpec(**lat, weights_of=1 if share and i > 0 else None))
+    return HybridArch(name=name, family="zadirax", hidden_size=width, vocab_size=vocab, layers=tuple(layers))
+
+
+HYBRID_PRESETS = {
+    # tests / CPU smoke: odd sizes on purpose (nothing a multiple of the MFMA tile)
+    "zadirax-tiny": lambda: _zadirax_preset("zadirax-tiny", 96, 300, 2, 3, 24, 136, 5, 2, 40, 56, 40, 8, share=True),
+    # layer sizes of a ~1.5B model (the width, head size, feed-forward and vocabulary of qwen2.5-1.5b)
+    "zadirax-1.5b": lambda: _zadirax_preset("zadirax-1.5b", 1536, 151936, 14, 12, 128, 8960, 32, 4, 2240, 512, 768, 64),
+}
+
+
+def resolve_arch(model_id: str, overrides: dict | None = None):
     """Resolve a model id / path to its architecture."""
     p = Path(os.path.expanduser(model_id))
     arch = None
     if p.is_dir() and (p / "config.json").exists():
-        arch = _from_hf_config(json.loads((p / "config.json").read_text()), p.name)
+        cfg = json.loads((p / "config.json").read_text())
+        parse = HYBRID_ARCHITECTURES.get(cfg.get("architecture"))
+        arch = parse(cfg, p.name) if parse else _from_hf_config(cfg, p.name)
     else:
         key = model_id.lower().split("/")[-1]
         key = key.replace("-instruct", "").replace("-awq", "").replace("_", "-")
+        if key in HYBRID_PRESETS:
+            arch = HYBRID_PRESETS[key]()
         for alias, preset in _ALIASES:
+            if arch is not None:
+                break
             if alias in key:
                 arch = PRESETS[preset]
                 break
     if arch is None:
-        raise ValueError(f"unknown model '{model_id}': pass a directory with config.json or one of {sorted(PRESETS)}")
+        raise ValueError(f"unknown model '{model_id}': pass a directory with config.json or one of "
+                         f"{sorted(PRESETS) + sorted(HYBRID_PRESETS)}")
     if overrides:
         arch = replace(arch, **overrides)
     return arch

@@ -1,0 +1,271 @@
+"""Ops of layered hybrid models (fp32 residual stream, bf16 or fp32 activations).
+
+Same dispatch rule as the rest of :mod:`vgate.ops`: GPU tensors go to the HIP kernels
+(csrc/kernels/gemm_any.hip, seq_elementwise.hip, latent_attn.hip, delta_rule.hip) and raise if the
+extension is missing; CPU tensors run the unfused torch forms below (the CPU device of tests).
+Everything the kernels compute in fp32 is fp32 here too; rows are rounded to the activation dtype
+at the same places.
+"""
+from __future__ import annotations
+
+import torch
+
+
+def _C():
+    from vgate import ops
+    return ops.native()
+
+
+class RowLinear:
+    """A linear layer kept row-major [N, K] (bf16 or fp32): the operand of :func:`gemm`.
+
+    ``w`` may be 3-D: one matrix per head (batched) or per expert (grouped). ``bias`` is fp32."""
+
+    def __init__(self, w: torch.Tensor, bias: torch.Tensor | None = None):
+        self.w = w.contiguous()
+        self.bias = bias.float().contiguous() if bias is not None else None
+        self.N, self.K = w.shape[-2], w.shape[-1]
+
+    def nbytes(self) -> int:
+        return self.w.numel() * self.w.element_size()
+
+
+ACT_NONE, ACT_SILU_MUL, ACT_CLAMPED_GLU, ACT_TANH = 0, 1, 2, 3
+
+
+def _act(g: torch.Tensor, u: torch.Tensor | None, act: int, limit: float, alpha: float) -> torch.Tensor:
+    if act == ACT_SILU_MUL:
+        return g * torch.sigmoid(g) * u
+    if act == ACT_CLAMPED_GLU:
+        g = g.clamp(max=limit)
+        u = u.clamp(-limit, limit)
+        return g * torch.sigmoid(alpha * g) * (u + 1.0)
+    if act == ACT_TANH:
+        return torch.tanh(g)
+    return g
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w2: torch.Tensor | None = None,
+         bias: torch.Tensor | None = None, gate: torch.Tensor | None = None, a_rows: torch.Tensor | None = None,
+         group_off: torch.Tensor | None = None, act: int = 0, limit: float = 0.0, alpha: float = 1.702) -> torch.Tensor:
+    """out = epi(a @ w^T): 2-D, batched (3-D a / w / out) or grouped (2-D a / out, 3-D w, device row
+    ranges ``group_off``; rows of a gathered through ``a_rows``). Epilogue: + bias, activation (pair
+    forms take ``w2``), * sigmoid(gate). fp32 accumulation; one rounding to out's dtype."""
+    if a.is_cuda:
+        _C().gemm_any(a, w, out, w2, bias, gate, a_rows, group_off, act, limit, alpha)
+        return out
+    af, wf = a.float(), w.float()
+    if group_off is not None:
+        off = group_off.tolist()
+        res = torch.zeros(out.shape, dtype=torch.float32)
+        for g in range(w.shape[0]):
+            lo, hi = off[g], off[g + 1]
+            if hi <= lo:
+                continue
+            rows = af[a_rows[lo:hi].long()] if a_rows is not None else af[lo:hi]
+            y = rows @ wf[g].t()
+            u = rows @ w2[g].float().t() if w2 is not None else None
+            res[lo:hi] = _act(y, u, act, limit, alpha)
+        out.copy_(res)
+        return out
+    M = out.shape[-2]
+    af = af[a_rows[:M].long()] if a_rows is not None else af[..., :M, :]
+    y = af @ wf.transpose(-1, -2)
+    if bias is not None:
+        y = y + bias
+    u = af @ w2.float().transpose(-1, -2) if w2 is not None else None
+    y = _act(y, u, act, limit, alpha)
+    if gate is not None:
+        y = y * torch.sigmoid(gate[..., :M, :].float())
+    out.copy_(y)
+    return out
+
+
+def norm_rows(x: torch.Tensor, w: torch.Tensor, eps: float, out: torch.Tensor, rows: torch.Tensor | None = None,
+              scalar: bool = False) -> torch.Tensor:
+    """out[m] = x[rows[m]] / sqrt(mean(x^2) + eps) * w (w fp32: one number if ``scalar``)."""
+    if x.is_cuda:
+        _C().norm_rows(x, w, eps, out, rows, scalar)
+        return out
+    xf = x.float()
+    xf = xf[rows.long()] if rows is not None else xf[: out.shape[0]]
+    y = xf * (1.0 / torch.sqrt(xf.pow(2).mean(-1, keepdim=True) + eps)) * w
+    out.copy_(y)
+    return out
+
+
+def embed_rows(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, prev: torch.Tensor | None = None) -> torch.Tensor:
+    """fp32 rows of the embedding table; ids < 0 name the previous step's sample prev[-id - 1]."""
+    if table.is_cuda:
+        _C().embed_rows(ids, table, out, prev)
+        return out
+    if prev is not None and bool((ids < 0).any()):
+        ids = torch.where(ids < 0, prev.to(ids.device)[(-ids - 1).clamp(min=0).long()], ids)
+    out.copy_(table[ids.long()].float())
+    return out
+
+
+def gated_residual(x, y1, g1=None, b1=None, y2=None, g2=None, b2=None) -> None:
+    """x += y1 * sigmoid(g1 + b1) [+ y2 * sigmoid(g2 + b2)] in fp32 (g: strided column views)."""
+    if x.is_cuda:
+        _C().gated_residual(x, y1, g1, b1, y2, g2, b2)
+        return
+    T = x.shape[0]
+    v = y1.float()
+    if g1 is not None:
+        v = v * torch.sigmoid(g1[:T].float() + (b1 if b1 is not None else 0.0))
+    if y2 is not None:
+        u = y2.float()
+        if g2 is not None:
+            u = u * torch.sigmoid(g2[:T].float() + (b2 if b2 is not None else 0.0))
+        v = v + u
+    x += v
+
+
+def rope_inv_freq(dims: int, base: float, device) -> torch.Tensor:
+    """f_i = base^(-2i / dims), i < dims / 2, in fp32."""
+    i = torch.arange(dims // 2, dtype=torch.float32)
+    return (base ** (-2.0 * i / dims)).to(torch.float32).to(device)
+
+
+def _rope_pairs(x: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor, dims: int) -> torch.Tensor:
+    """Rotate the leading ``dims`` entries of the last axis in interleaved pairs (2i, 2i + 1); fp32."""
+    y = x.clone()
+    if dims == 0:
+        return y
+    ang = pos.float()[:, None] * inv_freq[None]
+    shape = [x.shape[0]] + [1] * (x.dim() - 2) + [dims // 2]
+    c, s = torch.cos(ang).view(shape), torch.sin(ang).view(shape)
+    u, v = x[..., 0:dims:2], x[..., 1:dims:2]
+    y[..., 0:dims:2] = u * c - v * s
+    y[..., 1:dims:2] = v * c + u * s
+    return y
+
+
+def latent_write(kv, w, eps, positions, slots, inv_freq, rot_dims: int, cache, rank: int) -> None:
+    """cache[slot] = [rmsnorm(kv[:rank]) * w, rope(kv[rank:])] for every token with slot >= 0."""
+    if kv.is_cuda:
+        _C().latent_write(kv, w, eps, positions, slots, inv_freq, rot_dims, cache, rank)
+        return
+    x = kv.float()
+    c = x[:, :rank]
+    c = c * (1.0 / torch.sqrt(c.pow(2).mean(-1, keepdim=True) + eps)) * w
+    kr = _rope_pairs(x[:, rank:], positions, inv_freq, rot_dims)
+    row = torch.cat([c, kr], -1).to(cache.dtype)
+    ok = slots >= 0
+    cache.view(-1, cache.shape[-1])[slots[ok].long()] = row[ok]
+
+
+def latent_qrope(q, positions, inv_freq, rot_dims: int, qa, H: int, dim: int, rank: int, rot: int) -> None:
+    """qa[t, h, rank:] = rope(q[t, h, dim:])."""
+    if q.is_cuda:
+        _C().latent_qrope(q, positions, inv_freq, rot_dims, qa, H, dim, rank, rot)
+        return
+    T = q.shape[0]
+    qr = q.view(T, H, dim + rot)[..., dim:].float()
+    qa.view(T, H, rank + rot)[..., rank:] = _rope_pairs(qr, positions, inv_freq, rot_dims).to(qa.dtype)
+
+
+def latent_attn(qa, cache, block_tables, context_lens, query_start, ol, scale: float, H: int, rank: int, rot: int,
+                num_seqs: int | None = None) -> None:
+    """ol[t, h] = sum_j softmax_j(scale * qa[t, h] . cache_j) cache_j[:rank], j <= position(t)."""
+    if qa.is_cuda:
+        _C().latent_attn(qa, cache, block_tables, context_lens, query_start, ol, scale, H, rank, rot)
+        return
+    E = rank + rot
+    T = qa.numel() // (H * E)
+    q3 = qa.view(T, H, E).float()
+    o3 = ol.view(T, H, rank)
+    page = cache.shape[1]
+    S = block_tables.shape[0] if num_seqs is None else num_seqs
+    flat = cache.view(-1, E)
+    for s in range(S):
+        t0, t1 = int(query_start[s]), int(query_start[s + 1])
+        if t1 <= t0:
+            continue
+        ctx = int(context_lens[s])
+        j = torch.arange(ctx)
+        rows = flat[(block_tables[s].long()[j // page] * page + j % page)].float()
+        sc = torch.einsum("the,je->thj", q3[t0:t1], rows) * scale
+        pos = ctx - (t1 - t0) + torch.arange(t1 - t0)
+        sc = sc.masked_fill(j[None, None, :] > pos[:, None, None], float("-inf"))
+        o3[t0:t1] = torch.einsum("thj,jr->thr", torch.softmax(sc, -1), rows[:, :rank]).to(ol.dtype)
+
+
+def delta_rule(r, k, v, g, a, wl, w0, ab, nw, state, state_slots, context_lens, query_start, out,
+               decay_c: float, unit_eps: float, eps: float, num_seqs: int | None = None) -> None:
+    """Generalized delta rule over state slots (see csrc/kernels/delta_rule.hip); state [slots, H, D, D]."""
+    if r.is_cuda:
+        _C().delta_rule(r, k, v, g, a, wl, w0, ab, nw, state, state_slots, context_lens, query_start, out,
+                        decay_c, unit_eps, eps)
+        return
+    H, D = state.shape[1], state.shape[2]
+    S = state_slots.numel() if num_seqs is None else num_seqs
+    for s in range(S):
+        t0, t1 = int(query_start[s]), int(query_start[s + 1])
+        slot = int(state_slots[s])
+        if t1 <= t0 or slot < 0:
+            continue
+        pos0 = int(context_lens[s]) - (t1 - t0)
+        St = state[slot].clone() if pos0 > 0 else torch.zeros(H, D, D)
+
+        def hd(x):
+            return x[t0:t1].float().view(t1 - t0, H, D)
+
+        rr, kk, vv, gg = hd(r), hd(k), hd(v), hd(g)
+        w = torch.exp(-decay_c * torch.sigmoid(hd(wl) + w0.view(H, D)))
+        al = torch.sigmoid(hd(a) + ab.view(H, D))
+        u = kk * (1.0 / torch.sqrt(kk.pow(2).sum(-1, keepdim=True) + unit_eps))
+        for i in range(t1 - t0):
+            uS = torch.einsum("hk,hkv->hv", u[i], St)
+            St = w[i][:, :, None] * St - (al[i] * u[i])[:, :, None] * uS[:, None, :] + kk[i][:, :, None] * vv[i][:, None, :]
+            o = torch.einsum("hkv,hk->hv", St, rr[i])
+            o = o * (1.0 / torch.sqrt(o.pow(2).mean(-1, keepdim=True) + eps)) * nw.view(H, D) * torch.sigmoid(gg[i])
+            out[t0 + i] = o.reshape(H * D).to(out.dtype)
+        state[slot] = St
+
+
+def moe_route(z, corr, top: int, norm_eps: float, idx, wts) -> None:
+    """idx / wts [T, top]: largest sigmoid(z) + corr; weights sigmoid(z) of the chosen over their sum."""
+    if z.is_cuda:
+        _C().moe_route(z, corr, top, norm_eps, idx, wts)
+        return
+    s = torch.sigmoid(z)
+    choice = s + corr if corr is not None else s
+    # arg-max rounds, lowest index first on ties (the kernel's order)
+    c = choice.clone()
+    picks = []
+    for _ in range(top):
+        i = c.argmax(-1)
+        picks.append(i)
+        c.scatter_(1, i[:, None], float("-inf"))
+    ii = torch.stack(picks, 1)
+    ws = torch.gather(s, 1, ii)
+    idx.copy_(ii.int())
+    wts.copy_(ws / (ws.sum(-1, keepdim=True) + norm_eps))
+
+
+def moe_sort(idx, E: int, rows, pos, off) -> None:
+    """Group the (token, choice) pairs by expert: rows[p] = token, pos[t, c] = p, off[E + 1]."""
+    if idx.is_cuda:
+        _C().moe_sort(idx, E, rows, pos, off)
+        return
+    flat = idx.reshape(-1).long()
+    order = torch.argsort(flat, stable=True)
+    top = idx.shape[1]
+    rows.copy_((order // top).int())
+    p = torch.empty_like(order)
+    p[order] = torch.arange(order.numel())
+    pos.copy_(p.int().view(pos.shape))
+    cnt = torch.bincount(flat, minlength=E)
+    off.copy_(torch.cat([torch.zeros(1, dtype=torch.long), cnt.cumsum(0)]).int())
+
+
+def moe_combine(y, pos, wts, out) -> None:
+    """out[t] = sum_c wts[t, c] * y[pos[t, c]]."""
+    if y.is_cuda:
+        _C().moe_combine(y, pos, wts, out)
+        return
+    T, top = wts.shape
+    rows = y.float()[pos.view(T, top).long()]
+    out.copy_((rows * wts[:, :, None]).sum(1))

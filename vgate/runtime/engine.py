@@ -26,8 +26,8 @@ from dataclasses import dataclass, field
 import torch
 
 from vgate import ops
+from vgate.models import build_model
 from vgate.models.config import resolve_arch
-from vgate.models.transformer import DecoderModel
 from vgate.parallel.comm import TPGroup, init_tp
 from vgate.runtime.kv_cache import BLOCK_SIZE, KVCacheManager, allocate_kv_tensors
 from vgate.runtime.model_runner import ModelRunner
@@ -162,8 +162,11 @@ class LLMEngine:
             weights = os.path.expanduser(cfg.model)
         self.arch = resolve_arch(cfg.model, cfg.arch_overrides)
         t0 = time.perf_counter()
-        self.model = DecoderModel(self.arch, self.device, self.tp, cfg.quantization, cfg.seed, weights,
-                                  cfg.max_model_len)
+        self.model = build_model(self.arch, self.device, self.tp, cfg.quantization, cfg.seed, weights,
+                                 cfg.max_model_len, dtype=cfg.dtype)
+        # a model with per-sequence recurrent state: one state slot per live sequence, and no prefix
+        # reuse (a cached prefix holds keys, not the state its tokens left behind)
+        self.stateful = bool(getattr(self.model, "stateful", False))
         if self.device.type == "cuda":
             torch.cuda.synchronize()
         self.load_seconds = time.perf_counter() - t0
@@ -171,9 +174,13 @@ class LLMEngine:
         self.tp_self_check = "n/a"
         if self.tp.custom_ar is not None and cfg.tp_collective_self_check and not self.tp.simulated:
             self._collective_self_check()
-        self.kv_caches = allocate_kv_tensors(self.arch.num_layers, self.num_blocks, self.model.num_kv_heads_local,
-                                             self.arch.head_dim, self.device, block_size=cfg.block_size)
-        self.kvm = KVCacheManager(self.num_blocks, cfg.block_size, cfg.enable_prefix_caching)
+        if hasattr(self.model, "allocate_caches"):  # per-layer paged caches / state slots of its own shapes
+            self.kv_caches = self.model.allocate_caches(self.num_blocks, cfg.block_size, cfg.max_num_seqs)
+        else:
+            self.kv_caches = allocate_kv_tensors(self.arch.num_layers, self.num_blocks, self.model.num_kv_heads_local,
+                                                 self.arch.head_dim, self.device, block_size=cfg.block_size)
+        self.kvm = KVCacheManager(self.num_blocks, cfg.block_size, cfg.enable_prefix_caching and not self.stateful,
+                                  state_slots=cfg.max_num_seqs if self.stateful else 0)
         self.scheduler = Scheduler(self.kvm, cfg.max_num_seqs, cfg.max_num_batched_tokens, cfg.max_model_len)
         part = cfg.part_size or 512
         part = min(1024, max(32, (part + 31) // 32 * 32))
@@ -187,7 +194,7 @@ class LLMEngine:
                                   cfg.graph_token_buckets)
         self.prefill_plans: dict = {}
         self.plans_from_cache = False
-        if self.device.type == "cuda" and cfg.prefill_autotune:
+        if self.device.type == "cuda" and cfg.prefill_autotune and hasattr(self.model.layers[0], "qkv"):
             t1 = time.perf_counter()
             # prefill buckets (>= 128 rows) and the medium buckets of mixed prefill + decode steps
             ms = [t for t in self.runner.t_buckets if t > 16]  # (t_buckets end at max_num_batched_tokens)
@@ -207,7 +214,7 @@ class LLMEngine:
                      {f"{n}x{k}": p for (n, k), p in self.prefill_plans.items()})
         if gloo_tp and not eager:
             cap = self.tp.custom_bytes()
-            H, vloc = self.arch.hidden_size, self.model.shard.vocab
+            H, vloc = self.arch.hidden_size, self.model.shard.vocab  # (TP groups: transformer families only)
             self.runner.graph_ok = lambda T, S: T * H * 2 <= cap and S * vloc * 4 <= cap
         self.tokenizer = load_tokenizer(weights, cfg.tokenizer, self.arch)
         self.stats = EngineStats()
@@ -254,7 +261,10 @@ class LLMEngine:
     # ------------------------------------------------------------------ sizing
     def _size_kv(self) -> int:
         cfg = self.cfg
-        per_block = 2 * self.arch.num_layers * self.model.num_kv_heads_local * cfg.block_size * self.arch.head_dim * 2
+        if hasattr(self.model, "cache_bytes_per_block"):
+            per_block = self.model.cache_bytes_per_block(cfg.block_size)
+        else:
+            per_block = 2 * self.arch.num_layers * self.model.num_kv_heads_local * cfg.block_size * self.arch.head_dim * 2
         max_useful = cfg.max_num_seqs * ((cfg.max_model_len + cfg.block_size - 1) // cfg.block_size) * 2 + 64
         if cfg.num_kv_blocks:
             n = cfg.num_kv_blocks
@@ -518,6 +528,66 @@ class LLMEngine:
                 self.kvm.free(seq)
 
         return self.call(run), len(ids)
+
+    def replay_step(self, entries: list, end: list | None = None) -> torch.Tensor | None:
+        """Teacher-forced step: run given tokens instead of scheduled ones and return logits.
+
+        ``entries``: ``(request_id, tokens, want)`` per request — the request's next tokens (a prompt
+        portion or one token) and the places among them whose logits are asked for. All entries run
+        as ONE batch through the engine's own step path (pages and state slots from the cache
+        manager, step metadata, the model's forward and kernels) from the cache and state earlier
+        steps left; nothing is sampled. A request is admitted at its first entry and may skip steps.
+        ``end``: requests finished after this step; their pages and slot are given back.
+        Returns fp32 logits ``[sum(len(want)), vocab]`` in entry order (``None`` if nothing is wanted).
+        Not to be mixed with scheduled requests on the same engine."""
+        from vgate.runtime.scheduler import ScheduledBatch
+        self._drain_inflight()
+        items, rows, t = [], [], 0
+        for rid, tokens, want in entries:
+            seq = self._by_id.get(rid)
+            if seq is None:
+                seq = Sequence(request_id=rid, prompt_ids=[], params=SamplingParams(max_tokens=1))
+                seq.status = SeqStatus.RUNNING
+                self._by_id[rid] = seq
+                self.scheduler.running.append(seq)
+            n = len(tokens)
+            if n == 0:
+                continue
+            if seq.total_len + n > self.cfg.max_model_len:
+                raise RuntimeError(f"request {rid} exceeds max_model_len {self.cfg.max_model_len}")
+            seq.prompt_ids.extend(int(x) for x in tokens)
+            if not self.kvm.ensure(seq, n):
+                raise RuntimeError("replay_step: the cache pool has no free pages or state slots for this step")
+            items.append((seq, n))
+            rows.extend(t + int(w) for w in want)
+            t += n
+        logits = None
+        if items:
+            if t > self.runner.max_tokens or len(items) > self.runner.max_seqs:
+                raise RuntimeError("replay_step: the step exceeds max_num_batched_tokens / max_num_seqs")
+            batch = ScheduledBatch(items, t, t, 0, [])
+            hidden = self.runner.hidden_states(batch)
+            for seq, n in items:
+                seq.num_computed += n
+            self.stats.steps += 1
+            self.stats.prefill_tokens += t
+            if rows:
+                idx = torch.tensor(rows, dtype=torch.int32, device=self.device)
+                logits = self.model.logits_of(hidden, idx) if hasattr(self.model, "logits_of") else \
+                    self._logits_of_rows(hidden, idx)
+        for rid in end or []:
+            seq = self._by_id.pop(rid, None)
+            if seq is not None:
+                self.scheduler.finish(seq, "length")
+        return logits
+
+    def _logits_of_rows(self, hidden: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+        """Transformer families: final norm + LM head over chosen rows of the residual stream."""
+        m = self.model
+        lg = ops.linear(hidden, m.lm_head, out_f32=True, norm=(m.final_norm, self.arch.rms_eps), row_idx=rows) \
+            if hidden.is_cuda else ops.linear(ops.rmsnorm(hidden.index_select(0, rows.long()), m.final_norm,
+                                                          self.arch.rms_eps), m.lm_head, out_f32=True)
+        return lg[:, : self.arch.vocab_size]
 
     def run_until_idle(self, max_steps: int = 1_000_000) -> None:
         """Synchronous driver (tests / offline use): process everything queued."""

@@ -138,13 +138,20 @@ def make_allocator(num_blocks: int, block_size: int = BLOCK_SIZE, prefix_caching
 
 
 class KVCacheManager:
+    """Pages of the paged caches and, for models with recurrent state, one state slot per live
+    sequence. A slot is taken with a sequence's first pages and given back with them (finish,
+    preemption, abort), so every path that frees a sequence frees both; a reused slot is not
+    cleared here: a sequence's first step (position 0) starts its state from zero on the device."""
+
     def __init__(self, num_blocks: int, block_size: int = BLOCK_SIZE, prefix_caching: bool = False,
-                 prefer_native: bool = True):
+                 prefer_native: bool = True, state_slots: int = 0):
         self.block_size = block_size
         self.num_blocks = num_blocks
         self.prefix_caching = prefix_caching
         self.alloc = make_allocator(num_blocks, block_size, prefix_caching, prefer_native)
         self._hash = self.alloc.hash_block
+        self.num_state_slots = state_slots
+        self._free_slots = list(range(state_slots - 1, -1, -1))
 
     # ------------------------------------------------------------------ queries
     def num_free(self) -> int:
@@ -177,13 +184,20 @@ class KVCacheManager:
         seq.num_cached_prefix = seq.num_computed
         seq.hashed_blocks = len(seq.blocks)
 
+    def free_state_slots(self) -> int:
+        return len(self._free_slots)
+
     def ensure(self, seq: Sequence, n_new: int) -> bool:
         need = self.blocks_needed(seq, n_new)
-        if need == 0:
-            return True
-        if not self.alloc.can_allocate(need):
+        want_slot = self.num_state_slots > 0 and seq.state_slot < 0
+        if want_slot and not self._free_slots:
             return False
-        seq.blocks.extend(self.alloc.allocate(need))
+        if need and not self.alloc.can_allocate(need):
+            return False
+        if want_slot:
+            seq.state_slot = self._free_slots.pop()
+        if need:
+            seq.blocks.extend(self.alloc.allocate(need))
         return True
 
     def register_computed(self, seq: Sequence) -> None:
@@ -205,6 +219,9 @@ class KVCacheManager:
     def free(self, seq: Sequence) -> None:
         if seq.blocks:
             self.alloc.free(seq.blocks)
+        if seq.state_slot >= 0:
+            self._free_slots.append(seq.state_slot)
+            seq.state_slot = -1
         seq.blocks = []
         seq.block_hashes = []
         seq.hashed_blocks = 0

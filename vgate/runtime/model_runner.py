@@ -151,6 +151,7 @@ class ModelRunner:
         qs, cl, sidx = h["query_start"], h["context_lens"], h["sample_idx"]
         temp, topp, topk, seeds, offs = h["temperature"], h["top_p"], h["top_k"], h["seeds"], h["offsets"]
         tseq, tq0 = h["tile_seq"], h["tile_q0"]
+        sslot = h["state_slots"]
         bt = m.bt_host
         t = 0
         ntile = 0
@@ -180,6 +181,7 @@ class ModelRunner:
             bt[s, :nb] = blocks
             ctx = c0 + n
             cl[s] = ctx
+            sslot[s] = seq.state_slot
             t += n
             qs[s + 1] = t
             sidx[s] = t - 1
@@ -205,6 +207,7 @@ class ModelRunner:
         slots[t:T] = -1
         qs[ns + 1: S + 1] = t
         cl[ns:S] = 0
+        sslot[ns:S] = -1
         sidx[ns:S] = 0
         temp[ns:S] = 0.0
         topp[ns:S] = 1.0
@@ -553,6 +556,7 @@ class ModelRunner:
         h["slots"][:T] = -1
         h["query_start"][: S + 1] = 0
         h["context_lens"][:S] = 0
+        h["state_slots"][:S] = -1
         h["sample_idx"][:S] = 0
         h["temperature"][:S] = 0
         h["top_p"][:S] = 1

@@ -51,6 +51,8 @@ class Sequence:
     # device, not yet seen by the host) and the sample slot of the newest one
     pending: collections.deque = field(default_factory=collections.deque)
     pending_slot: int = -1
+    # models with recurrent state: the slot of the per-sequence state tensors (KVCacheManager), -1 = none
+    state_slot: int = -1
 
     @property
     def all_ids(self) -> list[int]:

@@ -38,6 +38,7 @@ class StepView:
     top_k: torch.Tensor
     seeds: torch.Tensor
     offsets: torch.Tensor
+    state_slots: torch.Tensor | None = None  # [S] state slot of each sequence (-1: none / padding)
     ring_slot: torch.Tensor | None = None  # [1]: slot of the pinned ring the step's sampled ids go to
     prev_tokens: torch.Tensor | None = None  # previous step's sampled ids (ids < 0 refer into it)
     num_tokens: int = 0
@@ -57,7 +58,8 @@ class StepMeta:
             ("ids", np.int32, self.T), ("positions", np.int32, self.T), ("slots", np.int32, self.T),
             ("query_start", np.int32, self.S + 1), ("context_lens", np.int32, self.S),
             ("tile_seq", np.int32, self.tiles), ("tile_q0", np.int32, self.tiles),
-            ("sample_idx", np.int32, self.S), ("ring_slot", np.int32, 4),
+            ("sample_idx", np.int32, self.S), ("state_slots", np.int32, self.S),
+            ("ring_slot", np.int32, 4),
             ("block_tables", np.int32, self.S * max_blocks),
         ]
         off = 0
@@ -123,5 +125,5 @@ class StepMeta:
             tile_seq=d["tile_seq"][:nt], tile_q0=d["tile_q0"][:nt],
             sample_idx=d["sample_idx"][:S], block_tables=d["block_tables"].view(self.S, self.max_blocks)[:S],
             temperature=d["temperature"][:S], top_p=d["top_p"][:S], top_k=d["top_k"][:S],
-            seeds=d["seeds"][:S], offsets=d["offsets"][:S], ring_slot=d["ring_slot"][:1],
+            seeds=d["seeds"][:S], offsets=d["offsets"][:S], state_slots=d["state_slots"][:S], ring_slot=d["ring_slot"][:1],
             prev_tokens=self.prev_tokens)
