@@ -22,9 +22,11 @@ import torch
 from vgate import ops
 from vgate.ops import seq
 
-# bf16 matrices whose shape the fragment-packed MFMA GEMMs take (N % 16, K % 32) run there; the rest
-# (and every fp32 matrix) through the row-major GEMM. "0" sends everything through the row-major one.
+# bf16 matrices in the shape range the fragment-packed MFMA GEMMs are exercised on (N and K multiples
+# of 64, K >= 512: the transformer families' projections) run there; the rest (and every fp32 matrix)
+# through the row-major GEMM. "0" sends everything through the row-major one.
 USE_PACKED = os.environ.get("VGATE_HYBRID_PACKED", "1") == "1"
+PACKED_MIN_K = 512
 
 
 class Proj:
@@ -34,8 +36,9 @@ class Proj:
         N, K = w.shape
         self.N, self.K, self.f32, self.silu_pair = N, K, f32, silu_pair
         dev = torch.device(device)
-        n_ok = (N // 2) % 8 == 0 if silu_pair else N % 16 == 0
-        self.packed = (USE_PACKED and allow_packed and not f32 and dev.type == "cuda" and n_ok and K % 32 == 0)
+        n_ok = (N // 2) % 64 == 0 if silu_pair else N % 64 == 0
+        self.packed = (USE_PACKED and allow_packed and not f32 and dev.type == "cuda" and n_ok and K % 64 == 0
+                       and K >= PACKED_MIN_K)
         if self.packed:
             self.lin = ops.Linear(w.to(dev, torch.bfloat16), kind="silu" if silu_pair else "plain")
             self.w = None

@@ -8,12 +8,37 @@ at the same places.
 """
 from __future__ import annotations
 
+import os
+
 import torch
+
+
+class _Traced:
+    """VGATE_SEQ_TRACE=1: print every kernel call (name, shapes) before it is launched and wait for
+    it, so a failing launch is named by the last line printed."""
+
+    def __init__(self, mod):
+        self._mod = mod
+
+    def __getattr__(self, name):
+        fn = getattr(self._mod, name)
+
+        def call(*a, **k):
+            shapes = [tuple(x.shape) if isinstance(x, torch.Tensor) else x for x in a]
+            print(f"[seq] {name} {shapes}", flush=True)
+            out = fn(*a, **k)
+            torch.cuda.synchronize()
+            return out
+        return call
+
+
+_TRACE = os.environ.get("VGATE_SEQ_TRACE", "0") == "1"
 
 
 def _C():
     from vgate import ops
-    return ops.native()
+    mod = ops.native()
+    return _Traced(mod) if _TRACE else mod
 
 
 class RowLinear:

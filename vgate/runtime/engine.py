@@ -575,6 +575,9 @@ class LLMEngine:
                 idx = torch.tensor(rows, dtype=torch.int32, device=self.device)
                 logits = self.model.logits_of(hidden, idx) if hasattr(self.model, "logits_of") else \
                     self._logits_of_rows(hidden, idx)
+            if self.device.type == "cuda":
+                # the step's metadata upload reads the pinned host buffer the next step rewrites
+                torch.cuda.current_stream(self.device).synchronize()
         for rid in end or []:
             seq = self._by_id.pop(rid, None)
             if seq is not None:
