@@ -355,7 +355,20 @@ def main():
     ap.add_argument("--switch-interval-us", type=float,
                     default=float(os.environ.get("VGATE_SWITCH_INTERVAL_US", "0")),
                     help="sys.setswitchinterval for the server process (0 = Python default 5 ms)")
+    ap.add_argument("--design-compare", action="store_true",
+                    help="instead of the serving benchmark: prefill / decode tokens/s of the Zadirax design beside a "
+                         "transformer of equal layer sizes (benchmarks/design_compare.py)")
+    ap.add_argument("--design-sizes", default="1024,1536", help="widths to compare (1024, 1536)")
+    ap.add_argument("--design-prefill", type=int, default=2048)
+    ap.add_argument("--design-batch", type=int, default=32)
+    ap.add_argument("--design-context", type=int, default=512)
     args = ap.parse_args()
+    if args.design_compare:
+        sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmarks"))
+        import design_compare
+        design_compare.main([int(x) for x in args.design_sizes.split(",")], args.design_prefill, args.design_batch,
+                            args.design_context)
+        return
     if args.switch_interval_us > 0:
         sys.setswitchinterval(args.switch_interval_us * 1e-6)
     if args.client_proc:

@@ -47,6 +47,13 @@ def config_b():
             "layers": [lat, _delta(1, 5, _moe(3, 1, 6, 0.7)), dict(lat, weights_of=0), _delta(3, 7, None)]}
 
 
+def config_c():
+    """Sizes in the range the fragment-packed MFMA GEMMs take (width 512, multiples of 64)."""
+    lat = _latent(4, 64, 64, 64, 192, 128, _moe(6, 2, 128, 3.0))
+    return {"architecture": "Zadirax", "width": 512, "vocab": 640, "norm": {"eps": 1e-6},
+            "layers": [_delta(4, 64, {"kind": "dense", "ff": 512}), lat, _delta(2, 128, {"kind": "dense", "ff": 512})]}
+
+
 def make_tensors(cfg: dict, seed: int, decay_rank: int = 3) -> dict:
     g = torch.Generator().manual_seed(seed)
     W, V = cfg["width"], cfg["vocab"]
@@ -95,7 +102,7 @@ def model_dir(tmp_path_factory, name: str):
     """(folder, config dict, fp32 tensors) of a named test model, written once per session."""
     if name not in _MODELS:
         from safetensors.torch import save_file
-        cfg = {"a": config_a, "b": config_b}[name]()
+        cfg = {"a": config_a, "b": config_b, "c": config_c}[name]()
         t = make_tensors(cfg, seed=11 if name == "a" else 23, decay_rank=3 if name == "a" else 2)
         d = tmp_path_factory.mktemp("zadirax_" + name)
         save_file({k: v.contiguous() for k, v in t.items()}, str(d / "model.safetensors"))
@@ -275,6 +282,24 @@ def test_generation_replays_graphs(tmp_path_factory):
         outs.append(done)
     assert eng.runner.graph_hits > hits
     assert outs[0] == outs[1]
+
+
+@pytest.mark.gpu
+def test_packed_gemm_path_matches_row_major_and_oracle(tmp_path_factory, monkeypatch):
+    """bf16 at sizes whose projections run on the fragment-packed MFMA GEMMs: same logits as with every
+    matrix on the row-major GEMM, and the oracle's; prompt portions, decoded tokens and a second request."""
+    from vgate.models import mixers
+    path, cfg, W = model_dir(tmp_path_factory, "c")
+    toks = tokens_of(cfg, 45, seed=5)
+    got = {}
+    for packed in (True, False):
+        monkeypatch.setattr(mixers, "USE_PACKED", packed)
+        eng = engine(path, "cuda", "bfloat16")
+        assert eng.model.layers[0].proj.packed == packed and eng.model.head.packed == packed
+        got[packed] = replay_all(eng, "p", toks, [30, 2, 9])
+        del eng
+    assert rel(got[True], got[False]) < 2e-2
+    assert rel(got[True], oracle_logits("c", cfg, W, toks)) < tol("bfloat16")
 
 
 def test_registry_and_config():

@@ -148,9 +148,14 @@ class HybridArch:
         return len(self.layers)
 
     def owner(self, i: int) -> int:
-        """Index of the layer whose tensors layer ``i`` runs with."""
-        w = self.layers[i].weights_of
-        return i if w is None else int(w)
+        """Index of the layer whose tensors layer ``i`` runs with (chains are followed)."""
+        seen = set()
+        while self.layers[i].weights_of is not None:
+            if i in seen:
+                raise ValueError(f"layer {i}: weights_of forms a cycle")
+            seen.add(i)
+            i = int(self.layers[i].weights_of)
+        return i
 
     def num_params(self) -> int:
         from vgate.models.mixers import layer_params
@@ -172,9 +177,6 @@ def _zadirax_from_config(cfg: dict, name: str) -> HybridArch:
             raise ValueError(f"layer {i}: weights_of {wo} names no other layer")
         layers.append(LayerSpec(kind=L["type"], mixer=dict(L["mixer"]), mlp=dict(L["mlp"]) if L.get("mlp") else None,
                                 weights_of=None if wo is None else int(wo)))
-    for i, L in enumerate(layers):
-        if L.weights_of is not None and layers[L.weights_of].weights_of is not None:
-            raise ValueError(f"layer {i}: weights_of must name a layer that owns its tensors")
     eos = cfg.get("eos_token_id", 2)
     return HybridArch(name=name, family="zadirax", hidden_size=int(cfg["width"]), vocab_size=int(cfg["vocab"]),
                       layers=tuple(layers), rms_eps=float(cfg["norm"]["eps"]),
@@ -204,6 +206,10 @@ def _zadirax_preset(name: str, width: int, vocab: int, pairs: int, heads: int, d
 HYBRID_PRESETS = {
     # tests / CPU smoke: odd sizes on purpose (nothing a multiple of the MFMA tile)
     "zadirax-tiny": lambda: _zadirax_preset("zadirax-tiny", 96, 300, 2, 3, 24, 136, 5, 2, 40, 56, 40, 8, share=True),
+    # 4-layer slices at the layer sizes of real models, for kernel / step benchmarks beside a transformer of
+    # equal width (benchmarks/design_compare.py)
+    "zadirax-bench-1024": lambda: _zadirax_preset("zadirax-bench-1024", 1024, 32000, 2, 8, 128, 4096, 8, 2, 2048, 256, 512, 64),
+    "zadirax-bench-1536": lambda: _zadirax_preset("zadirax-bench-1536", 1536, 32000, 2, 12, 128, 8960, 16, 4, 2240, 512, 768, 64),
     # layer sizes of a ~1.5B model (the width, head size, feed-forward and vocabulary of qwen2.5-1.5b)
     "zadirax-1.5b": lambda: _zadirax_preset("zadirax-1.5b", 1536, 151936, 14, 12, 128, 8960, 32, 4, 2240, 512, 768, 64),
 }

@@ -52,8 +52,8 @@ class LayerWeights:
             w = _pad8(w)
             parts.append(w)
             off += w.shape[0]
-        if off % 16:
-            parts.append(torch.zeros(16 - off % 16, width, dtype=parts[0].dtype))
+        if off % 64:  # whole 64-column tiles: the widest alignment any of the GEMMs asks for
+            parts.append(torch.zeros(64 - off % 64, width, dtype=parts[0].dtype))
         self.proj = Proj(torch.cat(parts), device, f32)
         del self.mixer.in_rows
 
@@ -145,13 +145,19 @@ class HybridModel:
         self.last_resid = x
         if return_hidden:
             return x
-        return self.logits_of(x, sv.sample_idx)
+        V = self.arch.vocab_size
+        if V % 4 == 0:
+            return self.logits_of(x, sv.sample_idx)
+        # the sampler reads rows of whole 16-B pieces: pad the row with -inf columns (never sampled)
+        buf = torch.full((sv.sample_idx.numel(), (V + 3) // 4 * 4), float("-inf"), dtype=torch.float32, device=dev)
+        self.logits_of(x, sv.sample_idx, out=buf[:, :V])
+        return buf
 
-    def logits_of(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+    def logits_of(self, x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         """fp32 logits [len(rows), vocab] of rows of the residual stream (final norm + head)."""
         hn = torch.empty(rows.numel(), x.shape[1], dtype=self.act_dtype, device=x.device)
         seq.norm_rows(x, self.final_norm, self.arch.rms_eps, hn, rows=rows, scalar=True)
-        return self.head(hn, out_f32=True)[:, : self.arch.vocab_size]
+        return self.head(hn, out_f32=True, out=out)[:, : self.arch.vocab_size]
 
 
 # ------------------------------------------------------------------------------------------ weights

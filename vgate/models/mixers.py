@@ -50,12 +50,13 @@ class Proj:
     def nbytes(self) -> int:
         return self.lin.nbytes() if self.packed else self.w.numel() * self.w.element_size()
 
-    def __call__(self, x: torch.Tensor, out_f32: bool = False, act: int = 0) -> torch.Tensor:
+    def __call__(self, x: torch.Tensor, out_f32: bool = False, act: int = 0, out: torch.Tensor | None = None) -> torch.Tensor:
         M = x.shape[0]
         if self.packed and act == 0:
-            return ops.linear(x, self.lin, out_f32=out_f32)
+            return ops.linear(x, self.lin, out=out, out_f32=out_f32)
         dt = torch.float32 if (out_f32 or self.f32) else torch.bfloat16
-        out = torch.empty(M, self.out_features, dtype=dt, device=x.device)
+        if out is None:
+            out = torch.empty(M, self.out_features, dtype=dt, device=x.device)
         if self.silu_pair:
             I = self.N // 2
             return seq.gemm(x, self.w[:I], out, w2=self.w[I:], act=seq.ACT_SILU_MUL)
