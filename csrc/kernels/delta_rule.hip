@@ -5,10 +5,16 @@
 //   u = k / sqrt(sum(k^2) + unit_eps)
 //   S <- diag(w) S - (a * u) (u^T S) + k v^T        (both correction terms read the old S)
 //   o  = S^T r;  out = o / rms(o) * nw * sigmoid(g)  (rms over the head)
-// One workgroup per (sequence, head), thread v owns column v of S in registers; the token's per-channel
-// vectors are shared through LDS. A sequence's tokens of the step (a prompt portion or one decoded
-// token) run in order from the slot's state; a portion that starts at position 0 starts from zero, so
-// a reused slot needs no clearing. The next token's inputs are loaded while the current one computes.
+// Three launches:
+//   prep   (token, head) parallel: the per-channel fp32 vectors {w, a * u, k, r} and u of every token.
+//   scan   the recurrence. Column v of S depends on no other column, so a head's D value columns are
+//          split into slices of 16 and every (sequence, head, slice) is one wave: lane = (key quarter,
+//          column), D / 4 state entries in registers, the two sums over keys (u^T S, r^T S) are
+//          D / 4 in-register FMAs + two cross-quarter lane swaps. Tokens are staged through LDS eight at
+//          a time, the next eight loaded into registers while the current ones compute. A sequence's
+//          tokens of the step run in order from the slot's state; a portion that starts at position 0
+//          starts from zero, so a reused slot needs no clearing.
+//   finish (token, head) parallel: head RMS norm, norm weight, output gate, store in the activation dtype.
 #include "common.h"
 #include "seq_launchers.h"
 
@@ -20,86 +26,190 @@ __device__ __forceinline__ float ldx(const void* p, int64_t i, int f32) {
 }
 __device__ __forceinline__ float sigm(float x) { return 1.f / (1.f + expf(-x)); }
 
-struct TokIn { float r, k, v, g, a, wl; };
-
-__device__ __forceinline__ TokIn load_tok(const DeltaArgs& p, int64_t t, int c, bool on) {
-  TokIn x{0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  if (on) {
-    const int64_t i = t * p.ld + c;
-    x.r = ldx(p.r, i, p.f32); x.k = ldx(p.k, i, p.f32); x.v = ldx(p.v, i, p.f32);
-    x.g = ldx(p.g, i, p.f32); x.a = ldx(p.a, i, p.f32);
-    x.wl = ldx(p.wl, t * p.ldw + c, p.f32);
+// one wave per (token, head): vec[t][h][d] = {w, a u, k, r}, un[t][h][d] = u
+__global__ __launch_bounds__(64) void delta_prep_kernel(DeltaArgs p, int T, float4* __restrict__ vec,
+                                                         float* __restrict__ un) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  if (t >= p.query_start[p.S]) return;  // padding rows of a graph bucket
+  const int D = p.D, lane = threadIdx.x;
+  float kk[2], rr[2], aa[2], ww[2];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int d = lane + 64 * i;
+    kk[i] = rr[i] = aa[i] = ww[i] = 0.f;
+    if (d < D) {
+      const int ch = h * D + d;
+      const int64_t ix = (int64_t)t * p.ld + ch;
+      kk[i] = ldx(p.k, ix, p.f32);
+      rr[i] = ldx(p.r, ix, p.f32);
+      aa[i] = sigm(ldx(p.a, ix, p.f32) + p.ab[ch]);
+      ww[i] = expf(-p.decay_c * sigm(ldx(p.wl, (int64_t)t * p.ldw + ch, p.f32) + p.w0[ch]));
+      ss = fmaf(kk[i], kk[i], ss);
+    }
   }
-  return x;
+  ss = wave_reduce_sum(ss);
+  const float inv = 1.f / sqrtf(ss + p.unit_eps);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int d = lane + 64 * i;
+    if (d < D) {
+      const float u = kk[i] * inv;
+      const int64_t o = ((int64_t)t * p.H + h) * D + d;
+      vec[o] = make_float4(ww[i], aa[i] * u, kk[i], rr[i]);
+      un[o] = u;
+    }
+  }
 }
 
-template <int DMAX>
-__global__ __launch_bounds__(DMAX) void delta_rule_kernel(DeltaArgs p) {
-  __shared__ float4 tok[DMAX];  // {w, a * u, k, r} per key channel
-  __shared__ float us[DMAX];
-  __shared__ float red[16];
-  const int s = blockIdx.x, h = blockIdx.y;
+constexpr int TC = 8;  // tokens staged per LDS buffer
+
+// lane = 16 * q + c: key quarter q (keys [q DQ', (q + 1) DQ') with DQ' = ceil(D / 4)), value column c0 + c
+template <int DQ>
+__global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float4* __restrict__ vec,
+                                                         const float* __restrict__ un, float* __restrict__ oraw) {
+  __shared__ float4 lv[2][TC][4 * DQ];
+  __shared__ float lu[2][TC][4 * DQ];
+  __shared__ float lvv[2][TC][16];  // the slice's value columns of each staged token
+  const int s = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * 16;
   const int slot = p.state_slots[s];
   const int t0 = p.query_start[s], t1 = p.query_start[s + 1];
   if (slot < 0 || t1 <= t0) return;
-  const int D = p.D;
-  const int v = threadIdx.x;
-  const bool on = v < D;
-  const int ch = h * D + v;
+  const int D = p.D, lane = threadIdx.x;
+  const int q = lane >> 4, c = c0 + (lane & 15);
+  const int dq = (D + 3) >> 2;         // keys per quarter at run time (<= DQ)
+  const int k0 = q * dq;
+  const bool con = c < D;
   const int pos0 = p.context_lens[s] - (t1 - t0);
   float* sp = p.state + ((int64_t)slot * p.H + h) * D * D;
-  float S[DMAX];
+  float S[DQ];
 #pragma unroll
-  for (int k = 0; k < DMAX; ++k) S[k] = (on && k < D && pos0 > 0) ? sp[(int64_t)k * D + v] : 0.f;
-  const float w0 = on ? p.w0[ch] : 0.f, ab = on ? p.ab[ch] : 0.f, nw = on ? p.nw[ch] : 0.f;
-  TokIn cur = load_tok(p, t0, ch, on);
-  for (int t = t0; t < t1; ++t) {
-    const TokIn nxt = load_tok(p, t + 1, ch, on && t + 1 < t1);
-    const float ksum = block_reduce_sum(cur.k * cur.k, red);
-    const float u = cur.k * (1.f / sqrtf(ksum + p.unit_eps));
-    const float w = expf(-p.decay_c * sigm(cur.wl + w0));
-    const float a = sigm(cur.a + ab);
-    if (on) {
-      tok[v] = make_float4(w, a * u, cur.k, cur.r);
-      us[v] = u;
-    }
-    __syncthreads();
-    float uS = 0.f;
+  for (int j = 0; j < DQ; ++j)
+    S[j] = (con && j < dq && k0 + j < D && pos0 > 0) ? sp[(int64_t)(k0 + j) * D + c] : 0.f;
+  // staging: a token's D channels are D float4 + D floats; lane l moves channels l, l + 64 of each token
+  float4 pv[TC][2];
+  float pu[TC][2];
+  float pvv[TC / 4];
+  auto fetch = [&](int tb) {
 #pragma unroll
-    for (int k = 0; k < DMAX; ++k)
-      if (k < D) uS = fmaf(us[k], S[k], uS);
-    float o = 0.f;
+    for (int i = 0; i < TC; ++i)
 #pragma unroll
-    for (int k = 0; k < DMAX; ++k)
-      if (k < D) {
-        const float4 c = tok[k];
-        S[k] = fmaf(c.z, cur.v, fmaf(-c.y, uS, c.x * S[k]));
-        o = fmaf(c.w, S[k], o);
+      for (int e = 0; e < 2; ++e) {
+        const int d = lane + 64 * e, t = tb + i;
+        const bool ok = d < D && t < t1;
+        const int64_t o = ((int64_t)(ok ? t : t0) * p.H + h) * D + (ok ? d : 0);
+        pv[i][e] = ok ? vec[o] : make_float4(0.f, 0.f, 0.f, 0.f);
+        pu[i][e] = ok ? un[o] : 0.f;
       }
-    if (!on) o = 0.f;
-    const float ss = block_reduce_sum(o * o, red);  // (its barriers also fence this token's LDS reads)
-    if (on) {
-      const float y = o * (1.f / sqrtf(ss / (float)D + p.eps)) * nw * sigm(cur.g);
+#pragma unroll
+    for (int e = 0; e < TC / 4; ++e) {  // TC x 16 values, lane -> (token, column)
+      const int ix = lane + 64 * e, t = tb + (ix >> 4), cc = c0 + (ix & 15);
+      pvv[e] = (t < t1 && cc < D) ? ldx(p.v, (int64_t)t * p.ld + h * D + cc, p.f32) : 0.f;
+    }
+  };
+  // LDS index of channel d: quarter-major, padded to DQ per quarter
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < TC; ++i)
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int d = lane + 64 * e;
+        if (d < D) {
+          const int li = (d / dq) * DQ + (d % dq);
+          lv[buf][i][li] = pv[i][e];
+          lu[buf][i][li] = pu[i][e];
+        }
+      }
+#pragma unroll
+    for (int e = 0; e < TC / 4; ++e) {
+      const int ix = lane + 64 * e;
+      lvv[buf][ix >> 4][ix & 15] = pvv[e];
+    }
+  };
+  fetch(t0);
+  put(0);
+  __syncthreads();
+  int buf = 0;
+  for (int tb = t0; tb < t1; tb += TC) {
+    const bool more = tb + TC < t1;
+    if (more) fetch(tb + TC);
+    const int nt = min(TC, t1 - tb);
+    for (int i = 0; i < nt; ++i) {
+      const float vv = lvv[buf][i][lane & 15];
+      const float4* tv = &lv[buf][i][q * DQ];
+      const float* tu = &lu[buf][i][q * DQ];
+      float uS = 0.f;
+#pragma unroll
+      for (int j = 0; j < DQ; ++j)
+        if (j < dq && k0 + j < D) uS = fmaf(tu[j], S[j], uS);
+      uS += xor16(uS);
+      uS += xor32(uS);
+      float o = 0.f;
+#pragma unroll
+      for (int j = 0; j < DQ; ++j)
+        if (j < dq && k0 + j < D) {
+          const float4 x = tv[j];  // {w, a u, k, r}
+          S[j] = fmaf(x.z, vv, fmaf(-x.y, uS, x.x * S[j]));
+          o = fmaf(x.w, S[j], o);
+        }
+      o += xor16(o);
+      o += xor32(o);
+      if (con && q == 0) oraw[(int64_t)(tb + i) * p.H * D + h * D + c] = o;
+    }
+    if (more) {
+      put(buf ^ 1);
+      __syncthreads();
+      buf ^= 1;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < DQ; ++j)
+    if (con && j < dq && k0 + j < D) sp[(int64_t)(k0 + j) * D + c] = S[j];
+}
+
+// one wave per (token, head)
+__global__ __launch_bounds__(64) void delta_finish_kernel(DeltaArgs p, const float* __restrict__ oraw) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  if (t >= p.query_start[p.S]) return;
+  const int D = p.D, lane = threadIdx.x;
+  float o[2];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int d = lane + 64 * i;
+    o[i] = d < D ? oraw[((int64_t)t * p.H + h) * D + d] : 0.f;
+    ss = fmaf(o[i], o[i], ss);
+  }
+  ss = wave_reduce_sum(ss);
+  const float inv = 1.f / sqrtf(ss / (float)D + p.eps);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int d = lane + 64 * i;
+    if (d < D) {
+      const int ch = h * D + d;
+      const float y = o[i] * inv * p.nw[ch] * sigm(ldx(p.g, (int64_t)t * p.ld + ch, p.f32));
       const int64_t oi = (int64_t)t * p.ldo + ch;
       if (p.f32) reinterpret_cast<float*>(p.out)[oi] = y;
       else reinterpret_cast<bf16_t*>(p.out)[oi] = f2bf(y);
     }
-    cur = nxt;
-  }
-  if (on) {
-#pragma unroll
-    for (int k = 0; k < DMAX; ++k)
-      if (k < D) sp[(int64_t)k * D + v] = S[k];
   }
 }
 
 }  // namespace
 
-void launch_delta_rule(const DeltaArgs& a, hipStream_t st) {
-  if (a.S <= 0 || a.H <= 0) return;
-  const dim3 grid(a.S, a.H);
-  if (a.D <= 64) hipLaunchKernelGGL(delta_rule_kernel<64>, grid, dim3(64), 0, st, a);
-  else hipLaunchKernelGGL(delta_rule_kernel<128>, grid, dim3(128), 0, st, a);
+// scratch: T * H * D * 6 floats ({w, a u, k, r}, u, raw o)
+void launch_delta_rule(const DeltaArgs& a, int T, float* scratch, hipStream_t st) {
+  if (a.S <= 0 || a.H <= 0 || T <= 0) return;
+  const int64_t n = (int64_t)T * a.H * a.D;
+  float4* vec = reinterpret_cast<float4*>(scratch);
+  float* un = scratch + 4 * n;
+  float* oraw = scratch + 5 * n;
+  hipLaunchKernelGGL(delta_prep_kernel, dim3(T, a.H), dim3(64), 0, st, a, T, vec, un);
+  const dim3 grid(a.S, a.H, (a.D + 15) / 16);
+  if (a.D <= 32) hipLaunchKernelGGL(delta_scan_kernel<8>, grid, dim3(64), 0, st, a, vec, un, oraw);
+  else if (a.D <= 64) hipLaunchKernelGGL(delta_scan_kernel<16>, grid, dim3(64), 0, st, a, vec, un, oraw);
+  else hipLaunchKernelGGL(delta_scan_kernel<32>, grid, dim3(64), 0, st, a, vec, un, oraw);
+  hipLaunchKernelGGL(delta_finish_kernel, dim3(T, a.H), dim3(64), 0, st, a, oraw);
 }
 
 }  // namespace vgate

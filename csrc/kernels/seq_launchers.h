@@ -68,7 +68,8 @@ struct DeltaArgs {
   void* out = nullptr; int64_t ldo = 0;
   int S = 0, H = 0, D = 0, f32 = 0;
 };
-void launch_delta_rule(const DeltaArgs& a, hipStream_t st);
+// T rows; scratch: T * H * D * 6 floats (the prepared per-channel vectors and the raw outputs)
+void launch_delta_rule(const DeltaArgs& a, int T, float* scratch, hipStream_t st);
 
 // idx, wts [T][top]: the `top` largest of sigmoid(z) + corr; wts = sigmoid(z) of the chosen / their sum
 void launch_moe_route(const float* z, const float* corr, int T, int E, int top, float norm_eps, int32_t* idx,

@@ -205,7 +205,7 @@ void latent_attn(const Tensor& qa, const Tensor& cache, const Tensor& block_tabl
 void delta_rule(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor& g, const Tensor& a, const Tensor& wl,
                 const Tensor& w0, const Tensor& ab, const Tensor& nw, Tensor& state, const Tensor& state_slots,
                 const Tensor& context_lens, const Tensor& query_start, Tensor& out, double decay_c, double unit_eps,
-                double eps) {
+                double eps, Tensor& scratch) {
   vgate::DeltaArgs p;
   p.f32 = act_f32(r, "r");
   TORCH_CHECK(state.is_cuda() && state.scalar_type() == torch::kFloat32 && state.is_contiguous() && state.dim() == 4 &&
@@ -231,8 +231,11 @@ void delta_rule(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor&
   p.context_lens = i32p(context_lens, "context_lens", p.S);
   p.query_start = i32p(query_start, "query_start", p.S + 1);  // values <= T: set by the step metadata
   p.out = out.data_ptr(); p.ldo = out.stride(0);
+  TORCH_CHECK(scratch.is_cuda() && scratch.scalar_type() == torch::kFloat32 && scratch.is_contiguous() &&
+              scratch.numel() >= 6 * T * HD, "delta_rule: scratch fp32 with T * H * D * 6 elements");
+  TORCH_CHECK((reinterpret_cast<uintptr_t>(scratch.data_ptr()) & 15) == 0, "delta_rule: scratch must be 16-B aligned");
   c10::DeviceGuard guard(r.device());
-  vgate::launch_delta_rule(p, cur_stream());
+  vgate::launch_delta_rule(p, (int)T, scratch.data_ptr<float>(), cur_stream());
 }
 
 void moe_route(const Tensor& z, const OptT& corr, int64_t top, double norm_eps, Tensor& idx, Tensor& wts) {

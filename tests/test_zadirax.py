@@ -299,7 +299,10 @@ def test_packed_gemm_path_matches_row_major_and_oracle(tmp_path_factory, monkeyp
         got[packed] = replay_all(eng, "p", toks, [30, 2, 9])
         del eng
     assert rel(got[True], got[False]) < 2e-2
-    assert rel(got[True], oracle_logits("c", cfg, W, toks)) < tol("bfloat16")
+    # (bf16 rounding alone moves this model's logits by ~0.09 of their size; fp32 below is the sharp check)
+    assert rel(got[True], oracle_logits("c", cfg, W, toks)) < 0.2
+    eng = engine(path, "cuda", "float32")
+    assert rel(replay_all(eng, "f", toks, [30, 2, 9]), oracle_logits("c", cfg, W, toks)) < tol("float32")
 
 
 def test_registry_and_config():

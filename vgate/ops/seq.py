@@ -221,8 +221,9 @@ def delta_rule(r, k, v, g, a, wl, w0, ab, nw, state, state_slots, context_lens, 
                decay_c: float, unit_eps: float, eps: float, num_seqs: int | None = None) -> None:
     """Generalized delta rule over state slots (see csrc/kernels/delta_rule.hip); state [slots, H, D, D]."""
     if r.is_cuda:
+        scratch = torch.empty(6 * r.shape[0] * r.shape[1], dtype=torch.float32, device=r.device)
         _C().delta_rule(r, k, v, g, a, wl, w0, ab, nw, state, state_slots, context_lens, query_start, out,
-                        decay_c, unit_eps, eps)
+                        decay_c, unit_eps, eps, scratch)
         return
     H, D = state.shape[1], state.shape[2]
     S = state_slots.numel() if num_seqs is None else num_seqs
