@@ -68,8 +68,12 @@ constexpr int TC = 8;  // tokens staged per LDS buffer
 template <int DQ>
 __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float4* __restrict__ vec,
                                                          const float* __restrict__ un, float* __restrict__ oraw) {
-  __shared__ float4 lv[2][TC][4 * DQ];
-  __shared__ float lu[2][TC][4 * DQ];
+  // quarter strides padded (DQ + 1 float4 / DQ + 4 floats): the four quarters' broadcast reads of one
+  // instruction fall into different LDS banks. Entries of channels past D are zeroed once and never
+  // written, so the token loops run DQ iterations with no bounds test (zeros leave S, u^T S and o alone).
+  constexpr int QV = DQ + 1, QU = DQ + 4;
+  __shared__ float4 lv[2][TC][4 * QV];
+  __shared__ float lu[2][TC][4 * QU];
   __shared__ float lvv[2][TC][16];  // the slice's value columns of each staged token
   const int s = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * 16;
   const int slot = p.state_slots[s];
@@ -115,9 +119,8 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float
       for (int e = 0; e < 2; ++e) {
         const int d = lane + 64 * e;
         if (d < D) {
-          const int li = (d / dq) * DQ + (d % dq);
-          lv[buf][i][li] = pv[i][e];
-          lu[buf][i][li] = pu[i][e];
+          lv[buf][i][(d / dq) * QV + (d % dq)] = pv[i][e];
+          lu[buf][i][(d / dq) * QU + (d % dq)] = pu[i][e];
         }
       }
 #pragma unroll
@@ -126,6 +129,9 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float
       lvv[buf][ix >> 4][ix & 15] = pvv[e];
     }
   };
+  for (int e = lane; e < 2 * TC * 4 * QV; e += 64) (&lv[0][0][0])[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int e = lane; e < 2 * TC * 4 * QU; e += 64) (&lu[0][0][0])[e] = 0.f;
+  __syncthreads();
   fetch(t0);
   put(0);
   __syncthreads();
@@ -136,22 +142,20 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float
     const int nt = min(TC, t1 - tb);
     for (int i = 0; i < nt; ++i) {
       const float vv = lvv[buf][i][lane & 15];
-      const float4* tv = &lv[buf][i][q * DQ];
-      const float* tu = &lu[buf][i][q * DQ];
+      const float4* tv = &lv[buf][i][q * QV];
+      const float* tu = &lu[buf][i][q * QU];
       float uS = 0.f;
 #pragma unroll
-      for (int j = 0; j < DQ; ++j)
-        if (j < dq && k0 + j < D) uS = fmaf(tu[j], S[j], uS);
+      for (int j = 0; j < DQ; ++j) uS = fmaf(tu[j], S[j], uS);
       uS += xor16(uS);
       uS += xor32(uS);
       float o = 0.f;
 #pragma unroll
-      for (int j = 0; j < DQ; ++j)
-        if (j < dq && k0 + j < D) {
-          const float4 x = tv[j];  // {w, a u, k, r}
-          S[j] = fmaf(x.z, vv, fmaf(-x.y, uS, x.x * S[j]));
-          o = fmaf(x.w, S[j], o);
-        }
+      for (int j = 0; j < DQ; ++j) {
+        const float4 x = tv[j];  // {w, a u, k, r}
+        S[j] = fmaf(x.z, vv, fmaf(-x.y, uS, x.x * S[j]));
+        o = fmaf(x.w, S[j], o);
+      }
       o += xor16(o);
       o += xor32(o);
       if (con && q == 0) oraw[(int64_t)(tb + i) * p.H * D + h * D + c] = o;

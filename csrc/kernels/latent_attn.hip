@@ -6,8 +6,19 @@
 //   ol[t][h]       = sum_j softmax_j(score) c_j
 // latent_write: RMS norm of the latent (fp32 statistics) + interleaved-pair rotation of the shared key
 // part + the paged store, one launch. Angles are position * inv_freq in fp32 with full-range sin / cos.
-// latent_attn: one workgroup per (token, group of heads); key tiles of 16 rows staged in LDS as fp32,
-// scores, running max / sum and the weighted latent sum all in fp32.
+// latent_attn, fp32 caches (and shapes the MFMA kernel does not take): one workgroup per (token, group
+// of heads); key tiles of 16 rows staged in LDS as fp32, scores, running max / sum and the weighted
+// latent sum all in fp32 FMA.
+// latent_attn, bf16 caches: MFMA kernel. Query rows are (token, head) pairs of one sequence, 16 per wave
+// (4 independent waves per workgroup), keys in tiles of 32 = two pages:
+//   S = Q K^T    v_mfma 16x16x32, Q fragments stationary in registers, K fragments (16 B of one cached
+//                row per lane) straight from the cache
+//   online softmax in fp32 (exp2 of log2(e)-scaled scores, per-lane partial row sums)
+//   O += P C     P goes C-layout -> A-layout through a 16 x 32 bf16 tile in LDS; the B operand needs
+//                eight consecutive KEYS of one latent column per lane, which the cache's second,
+//                transposed copy of the latent part ([page][column][16 keys], written by latent_write)
+//                delivers as one 16-B load: no transposition in the kernel
+// Waves of a workgroup never meet at a barrier (each loops to its own causal limit).
 #include "common.h"
 #include "seq_launchers.h"
 
@@ -23,7 +34,8 @@ __device__ __forceinline__ void stx(void* p, int64_t i, int f32, float v) {
 }
 
 __global__ __launch_bounds__(256) void latent_write_kernel(LatentArgs a, const void* __restrict__ kv, int64_t ldkv,
-                                                            const float* __restrict__ w, float eps) {
+                                                            const float* __restrict__ w, float eps,
+                                                            bf16_t* __restrict__ cache_t, int page) {
   __shared__ float red[16];
   const int t = blockIdx.x;
   const int slot = a.slots[t];
@@ -37,8 +49,12 @@ __global__ __launch_bounds__(256) void latent_write_kernel(LatentArgs a, const v
   }
   ss = block_reduce_sum(ss, red);
   const float inv = 1.f / sqrtf(ss / (float)a.rank + eps);
-  for (int c = threadIdx.x; c < a.rank; c += blockDim.x)
-    stx(a.cache, dst + c, a.f32, ldx(kv, src + c, a.f32) * inv * w[c]);
+  for (int c = threadIdx.x; c < a.rank; c += blockDim.x) {
+    const float v = ldx(kv, src + c, a.f32) * inv * w[c];
+    stx(a.cache, dst + c, a.f32, v);
+    if (cache_t != nullptr)  // [page][column][key in page]
+      cache_t[((int64_t)(slot / page) * a.rank + c) * page + slot % page] = f2bf(v);
+  }
   const float pos = (float)a.positions[t];
   for (int i = threadIdx.x; i < a.rot; i += blockDim.x) {
     float o;
@@ -178,11 +194,168 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(LatentArgs a, const vo
   }
 }
 
+
+// ---------------------------------------------------------------------------------- MFMA (bf16)
+__device__ __forceinline__ bf16x8 frag16(const bf16_t* rowp, int k, int K, bool valid) {
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (valid && k < K) {
+    const bf16_t* q = rowp + k;
+    if (k + 8 <= K && (reinterpret_cast<uintptr_t>(q) & 15) == 0) {
+      v = ld16(q);
+    } else {
+      uint32_t w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = (k + 2 * j < K) ? q[2 * j] : 0;
+        const uint32_t hi = (k + 2 * j + 1 < K) ? q[2 * j + 1] : 0;
+        w[j] = lo | (hi << 16);
+      }
+      v = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  }
+  return as_bf16x8(v);
+}
+
+__device__ __forceinline__ float group16_max(float v) {  // over the 16 lanes that share l >> 4
+  v = fmaxf(v, __shfl_xor(v, 8, 64)); v = fmaxf(v, __shfl_xor(v, 4, 64));
+  v = fmaxf(v, __shfl_xor(v, 2, 64)); v = fmaxf(v, __shfl_xor(v, 1, 64));
+  return v;
+}
+__device__ __forceinline__ float group16_sum(float v) {
+  v += __shfl_xor(v, 8, 64); v += __shfl_xor(v, 4, 64); v += __shfl_xor(v, 2, 64); v += __shfl_xor(v, 1, 64);
+  return v;
+}
+
+// NCT: 16-column tiles of the latent (rank <= 16 NCT); NQF: 32-wide fragments of a query row (E <= 32 NQF)
+template <int NCT, int NQF>
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, const bf16_t* __restrict__ qa, int H,
+                                                                float scale_log2e,
+                                                                const int32_t* __restrict__ block_tables,
+                                                                int max_blocks, int num_pages,
+                                                                const int32_t* __restrict__ context_lens,
+                                                                const int32_t* __restrict__ query_start, int S,
+                                                                const bf16_t* __restrict__ cache_t,
+                                                                bf16_t* __restrict__ ol) {
+  __shared__ __attribute__((aligned(16))) bf16_t pl[4][16][40];
+  const int E = a.rank + a.rot, KR = a.rank;
+  int s = -1, tile = 0, base = 0;
+  for (int i = 0; i < S; ++i) {  // (sequence, 64-row tile) of this workgroup
+    const int nt = ((query_start[i + 1] - query_start[i]) * H + 63) / 64;
+    if ((int)blockIdx.x < base + nt) { s = i; tile = blockIdx.x - base; break; }
+    base += nt;
+  }
+  if (s < 0) return;
+  const int wv = threadIdx.x >> 6, l = threadIdx.x & 63, lr = l & 15, lg = l >> 4;
+  const int t0 = query_start[s], ntok = query_start[s + 1] - t0;
+  const int pos0 = context_lens[s] - ntok;
+  const int nrows = ntok * H;
+  const int row0 = tile * 64 + wv * 16;
+  if (row0 >= nrows) return;
+  const bf16_t* cache = reinterpret_cast<const bf16_t*>(a.cache);
+  const int nqf = (E + 31) >> 5, nct = (KR + 15) >> 4;
+  // stationary Q fragments: A operand, lane holds Q[row lr][32 kk + 8 lg ..]
+  bf16x8 qf[NQF];
+  {
+    const int r = row0 + lr;
+    const bool ok = r < nrows;
+    const bf16_t* qrow = qa + ((int64_t)(t0 + (ok ? r / H : 0)) * H + (ok ? r % H : 0)) * E;
+#pragma unroll
+    for (int kk = 0; kk < NQF; ++kk) qf[kk] = frag16(qrow, 32 * kk + 8 * lg, E, ok && kk < nqf);
+  }
+  // C-layout rows of this lane: row0 + 4 lg + i; keys visible to each
+  int limit[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = row0 + 4 * lg + i;
+    limit[i] = r < nrows ? pos0 + r / H + 1 : 1;
+  }
+  const int last = min(row0 + 15, nrows - 1);
+  const int kmax = pos0 + last / H + 1;  // wave-uniform
+  float m[4], lsum[4];
+  f32x4 O[NCT];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { m[i] = -INFINITY; lsum[i] = 0.f; }
+#pragma unroll
+  for (int ct = 0; ct < NCT; ++ct) O[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int32_t* bt = block_tables + (int64_t)s * max_blocks;
+  for (int j0 = 0; j0 < kmax; j0 += 32) {
+    int pg0 = bt[j0 >> 4];
+    int pg1 = (j0 + 16 < kmax) ? bt[(j0 >> 4) + 1] : pg0;
+    pg0 = min(max(pg0, 0), num_pages - 1);
+    pg1 = min(max(pg1, 0), num_pages - 1);
+    f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = f32x4{0.f, 0.f, 0.f, 0.f};
+    const bf16_t* k0p = cache + ((int64_t)pg0 * 16 + lr) * E;
+    const bf16_t* k1p = cache + ((int64_t)pg1 * 16 + lr) * E;
+#pragma unroll
+    for (int kk = 0; kk < NQF; ++kk)
+      if (kk < nqf) {
+        s0 = mfma16(qf[kk], frag16(k0p, 32 * kk + 8 * lg, E, true), s0);
+        s1 = mfma16(qf[kk], frag16(k1p, 32 * kk + 8 * lg, E, true), s1);
+      }
+    float al[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float v0 = (j0 + lr < limit[i]) ? s0[i] * scale_log2e : -INFINITY;
+      const float v1 = (j0 + 16 + lr < limit[i]) ? s1[i] * scale_log2e : -INFINITY;
+      const float mnew = fmaxf(m[i], group16_max(fmaxf(v0, v1)));  // finite from the first tile on (key 0)
+      al[i] = exp2f(m[i] - mnew);
+      const float p0 = exp2f(v0 - mnew), p1 = exp2f(v1 - mnew);
+      lsum[i] = lsum[i] * al[i] + p0 + p1;
+      m[i] = mnew;
+      pl[wv][4 * lg + i][lr] = f2bf(p0);
+      pl[wv][4 * lg + i][16 + lr] = f2bf(p1);
+    }
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) O[ct][i] *= al[i];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's P tile is written (LDS is in order per wave)
+    const bf16x8 pf = as_bf16x8(*reinterpret_cast<const uint4*>(&pl[wv][lr][8 * lg]));
+    const int pgs = (lg >> 1) ? pg1 : pg0;
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct)
+      if (ct < nct) {
+        const int col = 16 * ct + lr;
+        uint4 b = make_uint4(0, 0, 0, 0);
+        if (col < KR) b = ld16(cache_t + (((int64_t)pgs * KR + col) * 16 + 8 * (lg & 1)));
+        O[ct] = mfma16(pf, as_bf16x8(b), O[ct]);
+      }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // P tile read before the next tile overwrites it
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float tot = group16_sum(lsum[i]);
+    const float inv = 1.f / tot;
+    const int r = row0 + 4 * lg + i;
+    if (r < nrows) {
+      bf16_t* orow = ol + ((int64_t)(t0 + r / H) * H + r % H) * KR;
+#pragma unroll
+      for (int ct = 0; ct < NCT; ++ct) {
+        const int col = 16 * ct + lr;
+        if (ct < nct && col < KR) orow[col] = f2bf(O[ct][i] * inv);
+      }
+    }
+  }
+}
+
+template <int NCT, int NQF>
+void launch_mfma(const LatentArgs& a, const void* qa, int H, float scale, const int32_t* block_tables, int max_blocks,
+                 int num_pages, const int32_t* context_lens, const int32_t* query_start, int S, const void* cache_t,
+                 void* ol, hipStream_t st) {
+  const int blocks = (a.T * H + 63) / 64 + S;
+  hipLaunchKernelGGL((latent_attn_mfma_kernel<NCT, NQF>), dim3(blocks), dim3(256), 0, st, a,
+                     reinterpret_cast<const bf16_t*>(qa), H, scale * 1.4426950408889634f, block_tables, max_blocks,
+                     num_pages, context_lens, query_start, S, reinterpret_cast<const bf16_t*>(cache_t),
+                     reinterpret_cast<bf16_t*>(ol));
+}
+
 }  // namespace
 
-void launch_latent_write(const LatentArgs& a, const void* kv, int64_t ldkv, const float* w, float eps, hipStream_t st) {
+void launch_latent_write(const LatentArgs& a, const void* kv, int64_t ldkv, const float* w, float eps, void* cache_t,
+                         int page, hipStream_t st) {
   if (a.T <= 0) return;
-  hipLaunchKernelGGL(latent_write_kernel, dim3(a.T), dim3(256), 0, st, a, kv, ldkv, w, eps);
+  hipLaunchKernelGGL(latent_write_kernel, dim3(a.T), dim3(256), 0, st, a, kv, ldkv, w, eps,
+                     reinterpret_cast<bf16_t*>(cache_t), page);
 }
 
 void launch_latent_qrope(const LatentArgs& a, const void* q, int H, int dim, void* qa, hipStream_t st) {
@@ -192,9 +365,18 @@ void launch_latent_qrope(const LatentArgs& a, const void* q, int H, int dim, voi
 
 void launch_latent_attn(const LatentArgs& a, const void* qa, int H, float scale, const int32_t* block_tables,
                         int max_blocks, int page, const int32_t* context_lens, const int32_t* query_start, int S,
-                        void* ol, hipStream_t st) {
+                        void* ol, const void* cache_t, int num_pages, hipStream_t st) {
   if (a.T <= 0 || S <= 0) return;
   const int E = a.rank + a.rot;
+  if (!a.f32 && cache_t != nullptr && page == 16 && a.rank <= 512 && E <= 640) {
+#define VG_LAT(NCT, NQF) launch_mfma<NCT, NQF>(a, qa, H, scale, block_tables, max_blocks, num_pages, context_lens, \
+                                               query_start, S, cache_t, ol, st)
+    if (a.rank <= 128 && E <= 192) VG_LAT(8, 6);
+    else if (a.rank <= 256 && E <= 384) VG_LAT(16, 12);
+    else VG_LAT(32, 20);
+#undef VG_LAT
+    return;
+  }
   int HC = H < 8 ? H : 8;
   while (HC > 1 && (HC * a.rank > 256 * MAXACC || (size_t)(HC + KT) * (E + 1) * 4 > 56 * 1024)) --HC;
   const size_t lds = ((size_t)(HC + KT) * (E + 1) + HC * KT + 3 * HC) * sizeof(float);

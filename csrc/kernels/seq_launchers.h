@@ -48,13 +48,15 @@ struct LatentArgs {
   int T = 0;
 };
 // cache[slot] = [rmsnorm(kv[:rank]) * w, rope(kv[rank:])]
-void launch_latent_write(const LatentArgs& a, const void* kv, int64_t ldkv, const float* w, float eps, hipStream_t st);
+// (cache_t: optional second, transposed bf16 copy of the latent part, [page][column][key in page])
+void launch_latent_write(const LatentArgs& a, const void* kv, int64_t ldkv, const float* w, float eps, void* cache_t,
+                         int page, hipStream_t st);
 // qa[t][h][rank:] = rope(q[t][h][dim:]) for q laid out [T][H][dim + rot], qa [T][H][rank + rot]
 void launch_latent_qrope(const LatentArgs& a, const void* q, int H, int dim, void* qa, hipStream_t st);
 // ol[t][h][:rank] = softmax_j(scale * qa[t][h] . cache[j]) . cache[j][:rank] over the causal keys
 void launch_latent_attn(const LatentArgs& a, const void* qa, int H, float scale, const int32_t* block_tables,
                         int max_blocks, int page, const int32_t* context_lens, const int32_t* query_start, int S,
-                        void* ol, hipStream_t st);
+                        void* ol, const void* cache_t, int num_pages, hipStream_t st);
 
 struct DeltaArgs {
   const void* r = nullptr; const void* k = nullptr; const void* v = nullptr; const void* g = nullptr;

@@ -154,7 +154,7 @@ vgate::LatentArgs latent_common(const Tensor& positions, const Tensor& inv_freq,
 }
 
 void latent_write(const Tensor& kv, const Tensor& w, double eps, const Tensor& positions, const Tensor& slots,
-                  const Tensor& inv_freq, int64_t rot_dims, Tensor& cache, int64_t rank) {
+                  const Tensor& inv_freq, int64_t rot_dims, Tensor& cache, int64_t rank, const OptT& cache_t) {
   const int f = act_f32(kv, "kv");
   TORCH_CHECK(kv.dim() == 2 && cache.dim() == 3 && cache.is_contiguous() && act_f32(cache, "cache") == f,
               "latent_write: kv [T, rank + rot], cache [pages, page, rank + rot] of one dtype");
@@ -164,8 +164,15 @@ void latent_write(const Tensor& kv, const Tensor& w, double eps, const Tensor& p
   a.slots = i32p(slots, "slots", kv.size(0));  // values < pages * page: written by the step's block tables
   a.cache = cache.data_ptr(); a.f32 = f;
   OptT wo(w);
+  void* ct = nullptr;
+  if (has(cache_t)) {
+    TORCH_CHECK(cache_t->is_cuda() && cache_t->scalar_type() == torch::kBFloat16 && cache_t->is_contiguous() &&
+                cache_t->numel() == cache.size(0) * cache.size(1) * rank, "latent_write: cache_t bf16 [pages, rank, page]");
+    ct = cache_t->data_ptr();
+  }
   c10::DeviceGuard guard(kv.device());
-  vgate::launch_latent_write(a, kv.data_ptr(), kv.stride(0), f32p(wo, "w", rank), (float)eps, cur_stream());
+  vgate::launch_latent_write(a, kv.data_ptr(), kv.stride(0), f32p(wo, "w", rank), (float)eps, ct, (int)cache.size(1),
+                             cur_stream());
 }
 
 void latent_qrope(const Tensor& q, const Tensor& positions, const Tensor& inv_freq, int64_t rot_dims, Tensor& qa,
@@ -181,7 +188,8 @@ void latent_qrope(const Tensor& q, const Tensor& positions, const Tensor& inv_fr
 }
 
 void latent_attn(const Tensor& qa, const Tensor& cache, const Tensor& block_tables, const Tensor& context_lens,
-                 const Tensor& query_start, Tensor& ol, double scale, int64_t H, int64_t rank, int64_t rot) {
+                 const Tensor& query_start, Tensor& ol, double scale, int64_t H, int64_t rank, int64_t rot,
+                 const OptT& cache_t) {
   const int f = act_f32(qa, "qa");
   const int64_t E = rank + rot;
   TORCH_CHECK(qa.is_contiguous() && qa.numel() % (H * E) == 0, "latent_attn: qa [T, H, rank + rot]");
@@ -197,9 +205,15 @@ void latent_attn(const Tensor& qa, const Tensor& cache, const Tensor& block_tabl
   const int32_t* bt = i32p(block_tables, "block_tables", 1);
   const int32_t* cl = i32p(context_lens, "context_lens", S);
   const int32_t* qs = i32p(query_start, "query_start", S + 1);
+  const void* ct = nullptr;
+  if (has(cache_t)) {
+    TORCH_CHECK(cache_t->is_cuda() && cache_t->scalar_type() == torch::kBFloat16 && cache_t->is_contiguous() &&
+                cache_t->numel() == cache.size(0) * cache.size(1) * rank, "latent_attn: cache_t bf16 [pages, rank, page]");
+    ct = cache_t->data_ptr();
+  }
   c10::DeviceGuard guard(qa.device());
   vgate::launch_latent_attn(a, qa.data_ptr(), (int)H, (float)scale, bt, (int)block_tables.size(1), (int)cache.size(1),
-                            cl, qs, (int)S, ol.data_ptr(), cur_stream());
+                            cl, qs, (int)S, ol.data_ptr(), ct, (int)cache.size(0), cur_stream());
 }
 
 void delta_rule(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor& g, const Tensor& a, const Tensor& wl,
@@ -290,9 +304,13 @@ void bind_seq(pybind11::module& m) {
   m.def("gated_residual", &gated_residual, "x += y1 * sigmoid(g1 + b1) + y2 * sigmoid(g2 + b2)", py::arg("x"),
         py::arg("y1"), py::arg("g1") = py::none(), py::arg("b1") = py::none(), py::arg("y2") = py::none(),
         py::arg("g2") = py::none(), py::arg("b2") = py::none());
-  m.def("latent_write", &latent_write, "latent norm + shared-key rotation + paged cache store");
+  m.def("latent_write", &latent_write, "latent norm + shared-key rotation + paged cache store", py::arg("kv"), py::arg("w"),
+        py::arg("eps"), py::arg("positions"), py::arg("slots"), py::arg("inv_freq"), py::arg("rot_dims"), py::arg("cache"),
+        py::arg("rank"), py::arg("cache_t") = py::none());
   m.def("latent_qrope", &latent_qrope, "rotate the rotated query part into the absorbed query buffer");
-  m.def("latent_attn", &latent_attn, "causal attention over the paged latent cache (absorbed projections)");
+  m.def("latent_attn", &latent_attn, "causal attention over the paged latent cache (absorbed projections)", py::arg("qa"),
+        py::arg("cache"), py::arg("block_tables"), py::arg("context_lens"), py::arg("query_start"), py::arg("ol"),
+        py::arg("scale"), py::arg("H"), py::arg("rank"), py::arg("rot"), py::arg("cache_t") = py::none());
   m.def("delta_rule", &delta_rule, "generalized delta rule recurrence over state slots + head norm + gate");
   m.def("moe_route", &moe_route, "sigmoid router: corrected top-k choice, normalised uncorrected weights");
   m.def("moe_sort", &moe_sort, "counting sort of (token, choice) pairs by expert");

@@ -367,11 +367,14 @@ def test_latent_attention_far_keys_and_edges(device, f32):
     bt = torch.zeros(1, 24, dtype=torch.int32)
     bt[0, :nblk] = perm.int()
     d = _dev(device)
-    ol = torch.zeros(nq, H, rank, dtype=dt, device=d)
-    seq.latent_attn(qa.to(d), cache.to(d), bt.to(d), torch.tensor([ctx], dtype=torch.int32, device=d),
-                    torch.tensor([0, nq], dtype=torch.int32, device=d), ol, 0.7, H, rank, rot)
     want = oracle_attend(qa.float(), rows.float(), rank, 0.7, ctx - nq)
-    assert rel(ol, want) < (2e-5 if f32 else 1e-2)
+    # bf16 on the GPU: also with the transposed copy of the latent part, which selects the MFMA kernel
+    copies = [None] if f32 or device == "cpu" else [None, cache[:, :, :rank].transpose(1, 2).contiguous().to(d)]
+    for cache_t in copies:
+        ol = torch.zeros(nq, H, rank, dtype=dt, device=d)
+        seq.latent_attn(qa.to(d), cache.to(d), bt.to(d), torch.tensor([ctx], dtype=torch.int32, device=d),
+                        torch.tensor([0, nq], dtype=torch.int32, device=d), ol, 0.7, H, rank, rot, cache_t=cache_t)
+        assert rel(ol, want) < (2e-5 if f32 else 1e-2), "mfma" if cache_t is not None else "fma"
     # the crafted keys matter: without the far key, or seeing the key one place too far, the answer moves
     no_far = rows.float().clone()
     no_far[far] -= 6.0 * probe

@@ -110,7 +110,18 @@ class LatentAttention:
                 "dkv.norm": (KR,), "uk": (H * D, KR), "uv": (H * V, KR), "g": (H * V, width), "o": (width, H * V)}
 
     def cache_shape(self, num_blocks: int, block_size: int, num_slots: int) -> tuple:
-        return (num_blocks, block_size, self.KR + self.R)
+        """One flat buffer per layer: rows [blocks, page, kv_rank + rot_dim], then (bf16) the transposed copy of
+        the latent part [blocks, kv_rank, page] that the MFMA attention kernel reads."""
+        self._page = block_size
+        return (num_blocks * block_size * (self.KR + self.R + (0 if self.f32 else self.KR)),)
+
+    def _views(self, cache: torch.Tensor):
+        E, block_size = self.KR + self.R, getattr(self, "_page", 16)
+        per = block_size * (E + (0 if self.f32 else self.KR))
+        nb = cache.numel() // per
+        rows = cache[: nb * block_size * E].view(nb, block_size, E)
+        tr = None if self.f32 else cache[nb * block_size * E:].view(nb, self.KR, block_size)
+        return rows, tr
 
     def cache_dtype(self):
         return torch.float32 if self.f32 else torch.bfloat16
@@ -126,14 +137,15 @@ class LatentAttention:
         cq = torch.empty(T, self.QR, dtype=dt, device=dev)
         seq.norm_rows(cols(P, "dq"), self.dq_norm, self.eps, cq)
         q = self.uq(cq)
+        cache, cache_t = self._views(cache)
         seq.latent_write(cols(P, "dkv"), self.dkv_norm, self.eps, sv.positions, sv.slots, self.inv_freq,
-                         self.rot_dims, cache, KR)
+                         self.rot_dims, cache, KR, cache_t=cache_t)
         qa = torch.empty(T, H, E, dtype=dt, device=dev)
         seq.gemm(q.view(T, H, D + R)[:, :, :D].permute(1, 0, 2), self.uk_t, qa[:, :, :KR].permute(1, 0, 2))
         seq.latent_qrope(q, sv.positions, self.inv_freq, self.rot_dims, qa, H, D, KR, R)
         ol = torch.empty(T, H, KR, dtype=dt, device=dev)
         seq.latent_attn(qa, cache, sv.block_tables, sv.context_lens, sv.query_start, ol, self.scale, H, KR, R,
-                        num_seqs=sv.num_seqs or None)
+                        num_seqs=sv.num_seqs or None, cache_t=cache_t)
         og = torch.empty(T, H, V, dtype=dt, device=dev)
         gate = cols(P, "g").unflatten(1, (H, V)).permute(1, 0, 2)
         seq.gemm(ol.permute(1, 0, 2), self.uv, og.permute(1, 0, 2), gate=gate)

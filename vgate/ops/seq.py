@@ -167,10 +167,12 @@ def _rope_pairs(x: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor, dims
     return y
 
 
-def latent_write(kv, w, eps, positions, slots, inv_freq, rot_dims: int, cache, rank: int) -> None:
-    """cache[slot] = [rmsnorm(kv[:rank]) * w, rope(kv[rank:])] for every token with slot >= 0."""
+def latent_write(kv, w, eps, positions, slots, inv_freq, rot_dims: int, cache, rank: int, cache_t=None) -> None:
+    """cache[slot] = [rmsnorm(kv[:rank]) * w, rope(kv[rank:])] for every token with slot >= 0.
+    ``cache_t`` (GPU, bf16): a second copy of the latent part laid out [page, column, key in page], the
+    operand layout of the MFMA attention kernel's weighted sum."""
     if kv.is_cuda:
-        _C().latent_write(kv, w, eps, positions, slots, inv_freq, rot_dims, cache, rank)
+        _C().latent_write(kv, w, eps, positions, slots, inv_freq, rot_dims, cache, rank, cache_t)
         return
     x = kv.float()
     c = x[:, :rank]
@@ -192,10 +194,11 @@ def latent_qrope(q, positions, inv_freq, rot_dims: int, qa, H: int, dim: int, ra
 
 
 def latent_attn(qa, cache, block_tables, context_lens, query_start, ol, scale: float, H: int, rank: int, rot: int,
-                num_seqs: int | None = None) -> None:
-    """ol[t, h] = sum_j softmax_j(scale * qa[t, h] . cache_j) cache_j[:rank], j <= position(t)."""
+                num_seqs: int | None = None, cache_t=None) -> None:
+    """ol[t, h] = sum_j softmax_j(scale * qa[t, h] . cache_j) cache_j[:rank], j <= position(t).
+    With ``cache_t`` (see :func:`latent_write`) bf16 caches run the MFMA kernel."""
     if qa.is_cuda:
-        _C().latent_attn(qa, cache, block_tables, context_lens, query_start, ol, scale, H, rank, rot)
+        _C().latent_attn(qa, cache, block_tables, context_lens, query_start, ol, scale, H, rank, rot, cache_t)
         return
     E = rank + rot
     T = qa.numel() // (H * E)
