@@ -226,7 +226,12 @@ __device__ __forceinline__ float group16_sum(float v) {
   return v;
 }
 
-// NCT: 16-column tiles of the latent (rank <= 16 NCT); NQF: 32-wide fragments of a query row (E <= 32 NQF)
+// NCT: 16-column tiles of the latent (rank <= 16 NCT); NQF: 32-wide fragments of a query row (E <= 32 NQF).
+// E % 8 == 0 (host-checked): every cache fragment is one unconditional 16-B load. Loads are issued in
+// groups (LG fragments, then their MFMAs) so a lone wave has several in flight; a fragment past the row's
+// end or the latent's last column is read from a clamped address: its partner (zero Q fragment) or its
+// output column (never stored) makes the value irrelevant, and cached values are always finite.
+constexpr int LG = 4;
 template <int NCT, int NQF>
 __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, const bf16_t* __restrict__ qa, int H,
                                                                 float scale_log2e,
@@ -287,11 +292,23 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
     const bf16_t* k0p = cache + ((int64_t)pg0 * 16 + lr) * E;
     const bf16_t* k1p = cache + ((int64_t)pg1 * 16 + lr) * E;
 #pragma unroll
-    for (int kk = 0; kk < NQF; ++kk)
-      if (kk < nqf) {
-        s0 = mfma16(qf[kk], frag16(k0p, 32 * kk + 8 * lg, E, true), s0);
-        s1 = mfma16(qf[kk], frag16(k1p, 32 * kk + 8 * lg, E, true), s1);
+    for (int k0 = 0; k0 < NQF; k0 += LG) {
+      if (k0 < nqf) {  // wave-uniform
+        uint4 b0[LG], b1[LG];
+#pragma unroll
+        for (int u = 0; u < LG; ++u) {
+          const int off = min(32 * (k0 + u) + 8 * lg, E - 8);
+          b0[u] = ld16(k0p + off);
+          b1[u] = ld16(k1p + off);
+        }
+#pragma unroll
+        for (int u = 0; u < LG; ++u)
+          if (k0 + u < NQF) {
+            s0 = mfma16(qf[k0 + u], as_bf16x8(b0[u]), s0);
+            s1 = mfma16(qf[k0 + u], as_bf16x8(b1[u]), s1);
+          }
       }
+    }
     float al[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -312,14 +329,18 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's P tile is written (LDS is in order per wave)
     const bf16x8 pf = as_bf16x8(*reinterpret_cast<const uint4*>(&pl[wv][lr][8 * lg]));
     const int pgs = (lg >> 1) ? pg1 : pg0;
+    const bf16_t* tp = cache_t + (int64_t)pgs * KR * 16 + 8 * (lg & 1);
 #pragma unroll
-    for (int ct = 0; ct < NCT; ++ct)
-      if (ct < nct) {
-        const int col = 16 * ct + lr;
-        uint4 b = make_uint4(0, 0, 0, 0);
-        if (col < KR) b = ld16(cache_t + (((int64_t)pgs * KR + col) * 16 + 8 * (lg & 1)));
-        O[ct] = mfma16(pf, as_bf16x8(b), O[ct]);
+    for (int c0 = 0; c0 < NCT; c0 += 2 * LG) {
+      if (c0 < nct) {  // wave-uniform
+        uint4 b[2 * LG];
+#pragma unroll
+        for (int u = 0; u < 2 * LG; ++u) b[u] = ld16(tp + (int64_t)min(16 * (c0 + u) + lr, KR - 1) * 16);
+#pragma unroll
+        for (int u = 0; u < 2 * LG; ++u)
+          if (c0 + u < NCT) O[c0 + u] = mfma16(pf, as_bf16x8(b[u]), O[c0 + u]);
       }
+    }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // P tile read before the next tile overwrites it
   }
 #pragma unroll
@@ -368,7 +389,7 @@ void launch_latent_attn(const LatentArgs& a, const void* qa, int H, float scale,
                         void* ol, const void* cache_t, int num_pages, hipStream_t st) {
   if (a.T <= 0 || S <= 0) return;
   const int E = a.rank + a.rot;
-  if (!a.f32 && cache_t != nullptr && page == 16 && a.rank <= 512 && E <= 640) {
+  if (!a.f32 && cache_t != nullptr && page == 16 && a.rank <= 512 && E <= 640 && E % 8 == 0 && E >= 8) {
 #define VG_LAT(NCT, NQF) launch_mfma<NCT, NQF>(a, qa, H, scale, block_tables, max_blocks, num_pages, context_lens, \
                                                query_start, S, cache_t, ol, st)
     if (a.rank <= 128 && E <= 192) VG_LAT(8, 6);
