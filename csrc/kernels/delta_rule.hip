@@ -8,9 +8,10 @@
 // Three launches:
 //   prep   (token, head) parallel: the per-channel fp32 vectors {w, a * u, k, r} and u of every token.
 //   scan   the recurrence. Column v of S depends on no other column, so a head's D value columns are
-//          split into slices of 16 and every (sequence, head, slice) is one wave: lane = (key quarter,
-//          column), D / 4 state entries in registers, the two sums over keys (u^T S, r^T S) are
-//          D / 4 in-register FMAs + two cross-quarter lane swaps. Tokens are staged through LDS eight at
+//          split into slices of 8 and every (sequence, head, slice) is one wave: lane = (key group of
+//          eight, column), D / 8 state entries in registers, the two sums over keys (u^T S, r^T S) are
+//          D / 8 in-register FMAs + three cross-group lane exchanges: the per-token dependency chain of
+//          a lone sequence's prefill is what bounds it, so the chain is kept short. Tokens are staged through LDS eight at
 //          a time, the next eight loaded into registers while the current ones compute. A sequence's
 //          tokens of the step run in order from the slot's state; a portion that starts at position 0
 //          starts from zero, so a reused slot needs no clearing.
@@ -64,7 +65,7 @@ __global__ __launch_bounds__(64) void delta_prep_kernel(DeltaArgs p, int T, floa
 
 constexpr int TC = 8;  // tokens staged per LDS buffer
 
-// lane = 16 * q + c: key quarter q (keys [q DQ', (q + 1) DQ') with DQ' = ceil(D / 4)), value column c0 + c
+// lane = 8 * q + c: key group q of 8 (keys [q DQ', (q + 1) DQ') with DQ' = ceil(D / 8)), value column c0 + c
 template <int DQ>
 __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float4* __restrict__ vec,
                                                          const float* __restrict__ un, float* __restrict__ oraw) {
@@ -72,16 +73,16 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float
   // instruction fall into different LDS banks. Entries of channels past D are zeroed once and never
   // written, so the token loops run DQ iterations with no bounds test (zeros leave S, u^T S and o alone).
   constexpr int QV = DQ + 1, QU = DQ + 4;
-  __shared__ float4 lv[2][TC][4 * QV];
-  __shared__ float lu[2][TC][4 * QU];
-  __shared__ float lvv[2][TC][16];  // the slice's value columns of each staged token
-  const int s = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * 16;
+  __shared__ float4 lv[2][TC][8 * QV];
+  __shared__ float lu[2][TC][8 * QU];
+  __shared__ float lvv[2][TC][8];  // the slice's value columns of each staged token
+  const int s = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * 8;
   const int slot = p.state_slots[s];
   const int t0 = p.query_start[s], t1 = p.query_start[s + 1];
   if (slot < 0 || t1 <= t0) return;
   const int D = p.D, lane = threadIdx.x;
-  const int q = lane >> 4, c = c0 + (lane & 15);
-  const int dq = (D + 3) >> 2;         // keys per quarter at run time (<= DQ)
+  const int q = lane >> 3, c = c0 + (lane & 7);
+  const int dq = (D + 7) >> 3;         // keys per group at run time (<= DQ)
   const int k0 = q * dq;
   const bool con = c < D;
   const int pos0 = p.context_lens[s] - (t1 - t0);
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float
   // staging: a token's D channels are D float4 + D floats; lane l moves channels l, l + 64 of each token
   float4 pv[TC][2];
   float pu[TC][2];
-  float pvv[TC / 4];
+  float pvv;
   auto fetch = [&](int tb) {
 #pragma unroll
     for (int i = 0; i < TC; ++i)
@@ -105,10 +106,9 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float
         pv[i][e] = ok ? vec[o] : make_float4(0.f, 0.f, 0.f, 0.f);
         pu[i][e] = ok ? un[o] : 0.f;
       }
-#pragma unroll
-    for (int e = 0; e < TC / 4; ++e) {  // TC x 16 values, lane -> (token, column)
-      const int ix = lane + 64 * e, t = tb + (ix >> 4), cc = c0 + (ix & 15);
-      pvv[e] = (t < t1 && cc < D) ? ldx(p.v, (int64_t)t * p.ld + h * D + cc, p.f32) : 0.f;
+    {  // TC x 8 values, lane -> (token, column)
+      const int t = tb + (lane >> 3), cc = c0 + (lane & 7);
+      pvv = (t < t1 && cc < D) ? ldx(p.v, (int64_t)t * p.ld + h * D + cc, p.f32) : 0.f;
     }
   };
   // LDS index of channel d: quarter-major, padded to DQ per quarter
@@ -123,14 +123,10 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float
           lu[buf][i][(d / dq) * QU + (d % dq)] = pu[i][e];
         }
       }
-#pragma unroll
-    for (int e = 0; e < TC / 4; ++e) {
-      const int ix = lane + 64 * e;
-      lvv[buf][ix >> 4][ix & 15] = pvv[e];
-    }
+    lvv[buf][lane >> 3][lane & 7] = pvv;
   };
-  for (int e = lane; e < 2 * TC * 4 * QV; e += 64) (&lv[0][0][0])[e] = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int e = lane; e < 2 * TC * 4 * QU; e += 64) (&lu[0][0][0])[e] = 0.f;
+  for (int e = lane; e < 2 * TC * 8 * QV; e += 64) (&lv[0][0][0])[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int e = lane; e < 2 * TC * 8 * QU; e += 64) (&lu[0][0][0])[e] = 0.f;
   __syncthreads();
   fetch(t0);
   put(0);
@@ -141,12 +137,13 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float
     if (more) fetch(tb + TC);
     const int nt = min(TC, t1 - tb);
     for (int i = 0; i < nt; ++i) {
-      const float vv = lvv[buf][i][lane & 15];
+      const float vv = lvv[buf][i][lane & 7];
       const float4* tv = &lv[buf][i][q * QV];
       const float* tu = &lu[buf][i][q * QU];
       float uS = 0.f;
 #pragma unroll
       for (int j = 0; j < DQ; ++j) uS = fmaf(tu[j], S[j], uS);
+      uS += __shfl_xor(uS, 8, 64);
       uS += xor16(uS);
       uS += xor32(uS);
       float o = 0.f;
@@ -156,6 +153,7 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float
         S[j] = fmaf(x.z, vv, fmaf(-x.y, uS, x.x * S[j]));
         o = fmaf(x.w, S[j], o);
       }
+      o += __shfl_xor(o, 8, 64);
       o += xor16(o);
       o += xor32(o);
       if (con && q == 0) oraw[(int64_t)(tb + i) * p.H * D + h * D + c] = o;
@@ -209,10 +207,10 @@ void launch_delta_rule(const DeltaArgs& a, int T, float* scratch, hipStream_t st
   float* un = scratch + 4 * n;
   float* oraw = scratch + 5 * n;
   hipLaunchKernelGGL(delta_prep_kernel, dim3(T, a.H), dim3(64), 0, st, a, T, vec, un);
-  const dim3 grid(a.S, a.H, (a.D + 15) / 16);
-  if (a.D <= 32) hipLaunchKernelGGL(delta_scan_kernel<8>, grid, dim3(64), 0, st, a, vec, un, oraw);
-  else if (a.D <= 64) hipLaunchKernelGGL(delta_scan_kernel<16>, grid, dim3(64), 0, st, a, vec, un, oraw);
-  else hipLaunchKernelGGL(delta_scan_kernel<32>, grid, dim3(64), 0, st, a, vec, un, oraw);
+  const dim3 grid(a.S, a.H, (a.D + 7) / 8);
+  if (a.D <= 32) hipLaunchKernelGGL(delta_scan_kernel<4>, grid, dim3(64), 0, st, a, vec, un, oraw);
+  else if (a.D <= 64) hipLaunchKernelGGL(delta_scan_kernel<8>, grid, dim3(64), 0, st, a, vec, un, oraw);
+  else hipLaunchKernelGGL(delta_scan_kernel<16>, grid, dim3(64), 0, st, a, vec, un, oraw);
   hipLaunchKernelGGL(delta_finish_kernel, dim3(T, a.H), dim3(64), 0, st, a, oraw);
 }
 
