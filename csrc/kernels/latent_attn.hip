@@ -18,7 +18,10 @@
 //                eight consecutive KEYS of one latent column per lane, which the cache's second,
 //                transposed copy of the latent part ([page][column][16 keys], written by latent_write)
 //                delivers as one 16-B load: no transposition in the kernel
-// Waves of a workgroup never meet at a barrier (each loops to its own causal limit).
+// Waves of a workgroup never meet at a barrier (each loops to its own causal limit), except for a
+// sequence whose rows fit one wave (a decoded token): there the four waves take every fourth key tile
+// of the same rows and merge their partial (max, sum, weighted latent) through LDS, so a lone token's
+// keys are streamed by four waves instead of one.
 #include "common.h"
 #include "seq_launchers.h"
 
@@ -242,6 +245,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
                                                                 const bf16_t* __restrict__ cache_t,
                                                                 bf16_t* __restrict__ ol) {
   __shared__ __attribute__((aligned(16))) bf16_t pl[4][16][40];
+  __shared__ float mrg_m[4][16], mrg_l[4][16];
+  __shared__ float mrg_o[16][16 * NCT];  // split mode: the merged weighted latent of the 16 rows
   const int E = a.rank + a.rot, KR = a.rank;
   int s = -1, tile = 0, base = 0;
   for (int i = 0; i < S; ++i) {  // (sequence, 64-row tile) of this workgroup
@@ -254,7 +259,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
   const int t0 = query_start[s], ntok = query_start[s + 1] - t0;
   const int pos0 = context_lens[s] - ntok;
   const int nrows = ntok * H;
-  const int row0 = tile * 64 + wv * 16;
+  const bool split = nrows <= 16;  // workgroup-uniform: one row tile, keys shared out over the four waves
+  const int row0 = split ? 0 : tile * 64 + wv * 16;
   if (row0 >= nrows) return;
   const bf16_t* cache = reinterpret_cast<const bf16_t*>(a.cache);
   const int nqf = (E + 31) >> 5, nct = (KR + 15) >> 4;
@@ -283,7 +289,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
 #pragma unroll
   for (int ct = 0; ct < NCT; ++ct) O[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int32_t* bt = block_tables + (int64_t)s * max_blocks;
-  for (int j0 = 0; j0 < kmax; j0 += 32) {
+  for (int j0 = split ? 32 * wv : 0; j0 < kmax; j0 += split ? 128 : 32) {
     int pg0 = bt[j0 >> 4];
     int pg1 = (j0 + 16 < kmax) ? bt[(j0 >> 4) + 1] : pg0;
     pg0 = min(max(pg0, 0), num_pages - 1);
@@ -314,9 +320,10 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
     for (int i = 0; i < 4; ++i) {
       const float v0 = (j0 + lr < limit[i]) ? s0[i] * scale_log2e : -INFINITY;
       const float v1 = (j0 + 16 + lr < limit[i]) ? s1[i] * scale_log2e : -INFINITY;
-      const float mnew = fmaxf(m[i], group16_max(fmaxf(v0, v1)));  // finite from the first tile on (key 0)
-      al[i] = exp2f(m[i] - mnew);
-      const float p0 = exp2f(v0 - mnew), p1 = exp2f(v1 - mnew);
+      const float mnew = fmaxf(m[i], group16_max(fmaxf(v0, v1)));
+      const float ms = (mnew == -INFINITY) ? 0.f : mnew;  // a row that has seen no key yet (split mode)
+      al[i] = exp2f(m[i] - ms);
+      const float p0 = exp2f(v0 - ms), p1 = exp2f(v1 - ms);
       lsum[i] = lsum[i] * al[i] + p0 + p1;
       m[i] = mnew;
       pl[wv][4 * lg + i][lr] = f2bf(p0);
@@ -343,9 +350,49 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // P tile read before the next tile overwrites it
   }
+  if (split) {
+    float f[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float tot = group16_sum(lsum[i]);
+      if (lr == 0) { mrg_m[wv][4 * lg + i] = m[i]; mrg_l[wv][4 * lg + i] = tot; }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 4 * lg + i;
+      float M = mrg_m[0][r];  // wave 0 always holds key 0: finite
+#pragma unroll
+      for (int w = 1; w < 4; ++w) M = fmaxf(M, mrg_m[w][r]);
+      float L = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) L += mrg_l[w][r] * exp2f(mrg_m[w][r] - M);
+      f[i] = exp2f(m[i] - M);     // a wave that saw no key: exp2(-inf) = 0
+      lsum[i] = L;                // the merged row sum (the same in every lane of the row)
+      m[i] = M;
+    }
+    for (int w = 0; w < 4; ++w) {  // waves add their scaled partials in turn
+      if (wv == w) {
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float* dst = &mrg_o[4 * lg + i][16 * ct + lr];
+            const float v = O[ct][i] * f[i];
+            *dst = (w == 0) ? v : *dst + v;
+          }
+      }
+      __syncthreads();
+    }
+    if (wv != 0) return;
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) O[ct][i] = mrg_o[4 * lg + i][16 * ct + lr];
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const float tot = group16_sum(lsum[i]);
+    const float tot = split ? lsum[i] : group16_sum(lsum[i]);
     const float inv = 1.f / tot;
     const int r = row0 + 4 * lg + i;
     if (r < nrows) {
