@@ -82,7 +82,11 @@ __device__ __forceinline__ bf16x8 load_frag(const bf16_t* rowp, int k, int K, bo
   return as_bf16x8(v);
 }
 
-template <int DUAL>
+// AL: K, the row strides and the batch strides are multiples of 8 elements and the bases 16-B aligned
+// (host-checked): every fragment is one unconditional 16-B load (rows / columns past the edge read a
+// clamped, valid row and are dropped at the store; k past K selects zero), two k-steps are loaded before
+// their MFMAs, so the loads of a wave overlap.
+template <int DUAL, bool AL>
 __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
   int grp, r0, rend;
   if (!locate_tile(p, blockIdx.y, grp, r0, rend)) return;
@@ -122,6 +126,39 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
       acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
       acc2[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+  if (AL) {
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    const int K = p.K;
+    for (int k0 = 0; k0 < K; k0 += 64) {
+      uint4 av[2][2], wv_[2][2], uv[2][2];
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        const int k = k0 + 32 * st + lk;
+        const int kc = min(k, K - 8);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          av[st][i] = ld16(arow[i] + kc);
+          wv_[st][i] = ld16(wrow[i] + kc);
+          if (DUAL) uv[st][i] = ld16(w2row[i] + kc);
+        }
+      }
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        const bool in = k0 + 32 * st + lk < K;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          if (!in) { av[st][i] = zero; wv_[st][i] = zero; if (DUAL) uv[st][i] = zero; }
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            acc[i][j] = mfma16(as_bf16x8(av[st][i]), as_bf16x8(wv_[st][j]), acc[i][j]);
+            if (DUAL) acc2[i][j] = mfma16(as_bf16x8(av[st][i]), as_bf16x8(uv[st][j]), acc2[i][j]);
+          }
+      }
+    }
+  } else
   for (int k0 = 0; k0 < p.K; k0 += 32) {
     const int k = k0 + lk;
     bf16x8 af[2], bfr[2], b2[2];
@@ -260,8 +297,13 @@ void launch_gemm_any(const AnyGemmArgs& g, hipStream_t st) {
     if (dual) hipLaunchKernelGGL((gemm_any_fma_kernel<bf16_t, 1>), grid, block, 0, st, g);
     else hipLaunchKernelGGL((gemm_any_fma_kernel<bf16_t, 0>), grid, block, 0, st, g);
   } else {
-    if (dual) hipLaunchKernelGGL((gemm_any_mfma_kernel<1>), grid, block, 0, st, g);
-    else hipLaunchKernelGGL((gemm_any_mfma_kernel<0>), grid, block, 0, st, g);
+    auto a16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    const bool al = g.K >= 8 && g.K % 8 == 0 && g.lda % 8 == 0 && g.ldw % 8 == 0 && g.a_bs % 8 == 0 &&
+                    g.w_bs % 8 == 0 && a16(g.a) && a16(g.w) && (!dual || a16(g.w2));
+    if (dual && al) hipLaunchKernelGGL((gemm_any_mfma_kernel<1, true>), grid, block, 0, st, g);
+    else if (dual) hipLaunchKernelGGL((gemm_any_mfma_kernel<1, false>), grid, block, 0, st, g);
+    else if (al) hipLaunchKernelGGL((gemm_any_mfma_kernel<0, true>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((gemm_any_mfma_kernel<0, false>), grid, block, 0, st, g);
   }
 }
 
