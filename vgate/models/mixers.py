@@ -85,14 +85,15 @@ class LatentAttention:
         self.KR, self.QR = int(m["kv_rank"]), int(m["q_rank"])
         self.scale = float(m["scale"])
         rot = m.get("rot") or {}
-        self.rot_dims = int(rot.get("dims", self.R))
-        if self.rot_dims > self.R or self.rot_dims % 2:
-            raise ValueError("latent_attention: rot.dims must be even and <= rot_dim")
+        dims = int(rot.get("dims", self.R))
+        if dims > self.R or dims < 0:
+            raise ValueError("latent_attention: rot.dims must be <= rot_dim")
+        self.rot_dims = 2 * (dims // 2)  # entries in rotated pairs (an odd last one passes unchanged)
         self.eps = eps
         self.f32 = f32
         dev = torch.device(device)
         H, D, R, V, KR = self.H, self.D, self.R, self.V, self.KR
-        self.inv_freq = seq.rope_inv_freq(self.rot_dims, float(rot.get("base", 10000.0)), dev)
+        self.inv_freq = seq.rope_inv_freq(dims, float(rot.get("base", 10000.0)), dev)  # base^(-2i / dims)
         self.in_rows = [("dq", tensors["dq"]), ("dkv", tensors["dkv"]), ("g", tensors["g"])]
         self.dq_norm, self.dkv_norm = _f32(tensors["dq.norm"], dev), _f32(tensors["dkv.norm"], dev)
         self.uq = Proj(tensors["uq"], dev, f32)
