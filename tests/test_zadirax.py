@@ -54,6 +54,14 @@ def config_c():
             "layers": [_delta(4, 64, {"kind": "dense", "ff": 512}), lat, _delta(2, 128, {"kind": "dense", "ff": 512})]}
 
 
+def config_d():
+    """Awkward sizes: a latent that is not a whole number of 16-column tiles, five heads, head sizes of the
+    recurrence that fill their key groups unevenly, every expert chosen, a vocabulary that is not a multiple of 4."""
+    lat = _latent(5, 24, 8, 40, 136, 48, _moe(3, 3, 24, 1.0), base=500.0)
+    return {"architecture": "Zadirax", "width": 72, "vocab": 101, "norm": {"eps": 1e-6},
+            "layers": [lat, _delta(3, 40, None), _delta(2, 100, {"kind": "dense", "ff": 50}), dict(lat, weights_of=0)]}
+
+
 def make_tensors(cfg: dict, seed: int, decay_rank: int = 3) -> dict:
     g = torch.Generator().manual_seed(seed)
     W, V = cfg["width"], cfg["vocab"]
@@ -102,7 +110,7 @@ def model_dir(tmp_path_factory, name: str):
     """(folder, config dict, fp32 tensors) of a named test model, written once per session."""
     if name not in _MODELS:
         from safetensors.torch import save_file
-        cfg = {"a": config_a, "b": config_b, "c": config_c}[name]()
+        cfg = {"a": config_a, "b": config_b, "c": config_c, "d": config_d}[name]()
         t = make_tensors(cfg, seed=11 if name == "a" else 23, decay_rank=3 if name == "a" else 2)
         d = tmp_path_factory.mktemp("zadirax_" + name)
         save_file({k: v.contiguous() for k, v in t.items()}, str(d / "model.safetensors"))
@@ -159,7 +167,7 @@ def replay_all(eng, rid, toks, cuts):
 # -------------------------------------------------------------------------------------------- engine
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("name", ["a", "b", "d"])
 def test_whole_prompt_matches_oracle(tmp_path_factory, device, dtype, name):
     path, cfg, W = model_dir(tmp_path_factory, name)
     toks = tokens_of(cfg, 37, seed=1)
@@ -236,6 +244,26 @@ def test_mixed_batches_and_reuse(tmp_path_factory, device, dtype):
     assert eng.kvm.num_free() == 8 and eng.kvm.free_state_slots() == 3
     for k, toks in reqs.items():
         assert rel(torch.cat(got[k]), oracle_logits("a", cfg, W, toks)) < tol(dtype), k
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_awkward_sizes_portions_and_batches(tmp_path_factory, device, dtype):
+    path, cfg, W = model_dir(tmp_path_factory, "d")
+    ta, tb = tokens_of(cfg, 45, seed=7), tokens_of(cfg, 21, seed=8)
+    eng = engine(path, device, dtype)
+    got_a, got_b = [], []
+    plan = [([0, 17], [0, 1]), ([17, 19], [1, 2]), ([19, 40], [2, 21]), ([40, 41], None), ([41, 45], None)]
+    for (a0, a1), br in plan:
+        entries = [("A", ta[a0:a1], list(range(a1 - a0)))]
+        if br:
+            entries.append(("B", tb[br[0]:br[1]], list(range(br[1] - br[0]))))
+        lg = eng.replay_step(entries, (["A"] if a1 == 45 else []) + (["B"] if br and br[1] == 21 else [])).float().cpu()
+        got_a.append(lg[: a1 - a0])
+        if br:
+            got_b.append(lg[a1 - a0:])
+    assert rel(torch.cat(got_a), oracle_logits("d", cfg, W, ta)) < tol(dtype)
+    assert rel(torch.cat(got_b), oracle_logits("d", cfg, W, tb)) < tol(dtype)
 
 
 @pytest.mark.parametrize("device", DEVICES)
