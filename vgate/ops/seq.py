@@ -41,20 +41,6 @@ def _C():
     return _Traced(mod) if _TRACE else mod
 
 
-class RowLinear:
-    """A linear layer kept row-major [N, K] (bf16 or fp32): the operand of :func:`gemm`.
-
-    ``w`` may be 3-D: one matrix per head (batched) or per expert (grouped). ``bias`` is fp32."""
-
-    def __init__(self, w: torch.Tensor, bias: torch.Tensor | None = None):
-        self.w = w.contiguous()
-        self.bias = bias.float().contiguous() if bias is not None else None
-        self.N, self.K = w.shape[-2], w.shape[-1]
-
-    def nbytes(self) -> int:
-        return self.w.numel() * self.w.element_size()
-
-
 ACT_NONE, ACT_SILU_MUL, ACT_CLAMPED_GLU, ACT_TANH = 0, 1, 2, 3
 
 
