@@ -86,13 +86,15 @@ __device__ __forceinline__ bf16x8 load_frag(const bf16_t* rowp, int k, int K, bo
 // (host-checked): every fragment is one unconditional 16-B load (rows / columns past the edge read a
 // clamped, valid row and are dropped at the store; k past K selects zero), two k-steps are loaded before
 // their MFMAs, so the loads of a wave overlap.
-template <int DUAL, bool AL>
+// NJ: 16-column tiles per wave (2: 64-column block tile; 4: 128-column block tile for wide outputs, which
+// loads 1.5x fewer fragment bytes per MFMA)
+template <int DUAL, bool AL, int NJ>
 __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
   int grp, r0, rend;
   if (!locate_tile(p, blockIdx.y, grp, r0, rend)) return;
   const int64_t b = blockIdx.z;
   const int64_t wsel = (p.group_off != nullptr) ? grp : b;
-  const int n0 = blockIdx.x * BN;
+  const int n0 = blockIdx.x * (32 * NJ);
   const int l = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int wm = wv & 1, wn = wv >> 1;
   const int lr = l & 15, lk = 8 * (l >> 4);
@@ -108,21 +110,21 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
     const int src = aval[i] ? (p.a_rows ? p.a_rows[m] : m) : 0;
     arow[i] = A + (int64_t)src * p.lda;
   }
-  const bf16_t* wrow[2];
-  const bf16_t* w2row[2];
-  bool wval[2];
+  const bf16_t* wrow[NJ];
+  const bf16_t* w2row[NJ];
+  bool wval[NJ];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int n = n0 + wn * 32 + j * 16 + lr;
+  for (int j = 0; j < NJ; ++j) {
+    const int n = n0 + wn * 16 * NJ + j * 16 + lr;
     wval[j] = n < p.N;
     wrow[j] = W + (int64_t)(wval[j] ? n : 0) * p.ldw;
     w2row[j] = DUAL ? W2 + (int64_t)(wval[j] ? n : 0) * p.ldw : nullptr;
   }
-  f32x4 acc[2][2], acc2[2][2];
+  f32x4 acc[2][NJ], acc2[2][NJ];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
       acc2[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -130,29 +132,30 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
     const uint4 zero = make_uint4(0, 0, 0, 0);
     const int K = p.K;
     for (int k0 = 0; k0 < K; k0 += 64) {
-      uint4 av[2][2], wv_[2][2], uv[2][2];
+      uint4 av[2][2], wv_[2][NJ], uv[2][NJ];
 #pragma unroll
       for (int st = 0; st < 2; ++st) {
         const int k = k0 + 32 * st + lk;
         const int kc = min(k, K - 8);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          av[st][i] = ld16(arow[i] + kc);
-          wv_[st][i] = ld16(wrow[i] + kc);
-          if (DUAL) uv[st][i] = ld16(w2row[i] + kc);
+        for (int i = 0; i < 2; ++i) av[st][i] = ld16(arow[i] + kc);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+          wv_[st][j] = ld16(wrow[j] + kc);
+          if (DUAL) uv[st][j] = ld16(w2row[j] + kc);
         }
       }
 #pragma unroll
       for (int st = 0; st < 2; ++st) {
         const bool in = k0 + 32 * st + lk < K;
+        if (!in) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          if (!in) { av[st][i] = zero; wv_[st][i] = zero; if (DUAL) uv[st][i] = zero; }
+          for (int i = 0; i < 2; ++i) av[st][i] = zero;  // a zero A fragment zeroes the product
         }
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j) {
+          for (int j = 0; j < NJ; ++j) {
             acc[i][j] = mfma16(as_bf16x8(av[st][i]), as_bf16x8(wv_[st][j]), acc[i][j]);
             if (DUAL) acc2[i][j] = mfma16(as_bf16x8(av[st][i]), as_bf16x8(uv[st][j]), acc2[i][j]);
           }
@@ -161,18 +164,18 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
   } else
   for (int k0 = 0; k0 < p.K; k0 += 32) {
     const int k = k0 + lk;
-    bf16x8 af[2], bfr[2], b2[2];
+    bf16x8 af[2], bfr[NJ], b2[NJ];
 #pragma unroll
     for (int i = 0; i < 2; ++i) af[i] = load_frag(arow[i], k, p.K, aval[i]);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       bfr[j] = load_frag(wrow[j], k, p.K, wval[j]);
       if (DUAL) b2[j] = load_frag(w2row[j], k, p.K, wval[j]);
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         acc[i][j] = mfma16(af[i], bfr[j], acc[i][j]);
         if (DUAL) acc2[i][j] = mfma16(af[i], b2[j], acc2[i][j]);
       }
@@ -180,8 +183,8 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int n = n0 + wn * 32 + j * 16 + lr;
+    for (int j = 0; j < NJ; ++j) {
+      const int n = n0 + wn * 16 * NJ + j * 16 + lr;
       if (n >= p.N) continue;
       const float bias = p.bias ? p.bias[n] : 0.f;
 #pragma unroll
@@ -300,10 +303,14 @@ void launch_gemm_any(const AnyGemmArgs& g, hipStream_t st) {
     auto a16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     const bool al = g.K >= 8 && g.K % 8 == 0 && g.lda % 8 == 0 && g.ldw % 8 == 0 && g.a_bs % 8 == 0 &&
                     g.w_bs % 8 == 0 && a16(g.a) && a16(g.w) && (!dual || a16(g.w2));
-    if (dual && al) hipLaunchKernelGGL((gemm_any_mfma_kernel<1, true>), grid, block, 0, st, g);
-    else if (dual) hipLaunchKernelGGL((gemm_any_mfma_kernel<1, false>), grid, block, 0, st, g);
-    else if (al) hipLaunchKernelGGL((gemm_any_mfma_kernel<0, true>), grid, block, 0, st, g);
-    else hipLaunchKernelGGL((gemm_any_mfma_kernel<0, false>), grid, block, 0, st, g);
+    const bool wide = al && g.N >= 512 && g.M >= 256;  // enough 64 x 128 tiles to fill the chip
+    const dim3 gridw((g.N + 127) / 128, mt, g.batch);
+    if (dual && wide) hipLaunchKernelGGL((gemm_any_mfma_kernel<1, true, 4>), gridw, block, 0, st, g);
+    else if (wide) hipLaunchKernelGGL((gemm_any_mfma_kernel<0, true, 4>), gridw, block, 0, st, g);
+    else if (dual && al) hipLaunchKernelGGL((gemm_any_mfma_kernel<1, true, 2>), grid, block, 0, st, g);
+    else if (dual) hipLaunchKernelGGL((gemm_any_mfma_kernel<1, false, 2>), grid, block, 0, st, g);
+    else if (al) hipLaunchKernelGGL((gemm_any_mfma_kernel<0, true, 2>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((gemm_any_mfma_kernel<0, false, 2>), grid, block, 0, st, g);
   }
 }
 

@@ -527,6 +527,16 @@ def test_row_major_gemm_forms(device, f32):
     out = torch.empty(70, 29, dtype=dt, device=d)
     seq.gemm(a.to(d), w.to(d), out, act=seq.ACT_TANH)
     assert rel(out, torch.tanh(a.float() @ w.float().T)) < t
+    # wide aligned outputs (the 128-column block tile on the GPU), single matrix + bias and a SiLU pair
+    a2 = torch.randn(300, 72, generator=g).to(dt)
+    w2a, w2b = (torch.randn(520, 72, generator=g) / 8).to(dt), (torch.randn(520, 72, generator=g) / 8).to(dt)
+    bias = torch.randn(520, generator=g)
+    o2 = torch.empty(300, 520, dtype=dt, device=d)
+    seq.gemm(a2.to(d), w2a.to(d), o2, bias=bias.to(d))
+    assert rel(o2, a2.float() @ w2a.float().T + bias) < t
+    seq.gemm(a2.to(d), w2a.to(d), o2, w2=w2b.to(d), act=seq.ACT_SILU_MUL)
+    ga = a2.float() @ w2a.float().T
+    assert rel(o2, ga * oracle.sigmoid(ga) * (a2.float() @ w2b.float().T)) < t
     # per head, reading and writing slices of wider rows
     q = torch.randn(9, 3, 11, generator=g).to(dt)
     wh = torch.randn(3, 6, 7, generator=g).to(dt)
