@@ -136,7 +136,11 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float
     const bool more = tb + TC < t1;
     if (more) fetch(tb + TC);
     const int nt = min(TC, t1 - tb);
-    for (int i = 0; i < nt; ++i) {
+    // unrolled over the staged tokens: the LDS reads of token i + 1 do not depend on token i's state, so
+    // they can be issued under its FMAs and lane exchanges
+#pragma unroll
+    for (int i = 0; i < TC; ++i) {
+      if (i >= nt) break;
       const float vv = lvv[buf][i][lane & 7];
       const float4* tv = &lv[buf][i][q * QV];
       const float* tu = &lu[buf][i][q * QU];
