@@ -136,24 +136,34 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float
     const bool more = tb + TC < t1;
     if (more) fetch(tb + TC);
     const int nt = min(TC, t1 - tb);
-    // unrolled over the staged tokens: the LDS reads of token i + 1 do not depend on token i's state, so
-    // they can be issued under its FMAs and lane exchanges
+    // unrolled over the staged tokens, with token i + 1's vectors read from LDS into a second register
+    // set before token i's FMAs and lane exchanges (they do not depend on the state)
+    float4 xv[2][DQ];
+    float xu[2][DQ], xvv[2];
+    auto grab = [&](int i, int r) {
+      const float4* tv = &lv[buf][i][q * QV];
+      const float* tu = &lu[buf][i][q * QU];
+#pragma unroll
+      for (int j = 0; j < DQ; ++j) { xv[r][j] = tv[j]; xu[r][j] = tu[j]; }
+      xvv[r] = lvv[buf][i][lane & 7];
+    };
+    grab(0, 0);
 #pragma unroll
     for (int i = 0; i < TC; ++i) {
       if (i >= nt) break;
-      const float vv = lvv[buf][i][lane & 7];
-      const float4* tv = &lv[buf][i][q * QV];
-      const float* tu = &lu[buf][i][q * QU];
+      if (i + 1 < TC) grab(i + 1, (i + 1) & 1);  // (past nt: stale but finite LDS, never used)
+      const int r = i & 1;
+      const float vv = xvv[r];
       float uS = 0.f;
 #pragma unroll
-      for (int j = 0; j < DQ; ++j) uS = fmaf(tu[j], S[j], uS);
+      for (int j = 0; j < DQ; ++j) uS = fmaf(xu[r][j], S[j], uS);
       uS += __shfl_xor(uS, 8, 64);
       uS += xor16(uS);
       uS += xor32(uS);
       float o = 0.f;
 #pragma unroll
       for (int j = 0; j < DQ; ++j) {
-        const float4 x = tv[j];  // {w, a u, k, r}
+        const float4 x = xv[r][j];  // {w, a u, k, r}
         S[j] = fmaf(x.z, vv, fmaf(-x.y, uS, x.x * S[j]));
         o = fmaf(x.w, S[j], o);
       }
