@@ -26,6 +26,10 @@ __device__ __forceinline__ float ldx(const void* p, int64_t i, int f32) {
   return f32 ? reinterpret_cast<const float*>(p)[i] : bf2f(reinterpret_cast<const bf16_t*>(p)[i]);
 }
 __device__ __forceinline__ float sigm(float x) { return 1.f / (1.f + expf(-x)); }
+// lane l gets lane l ^ 8's value: a rotation by 8 inside each row of 16 lanes (DPP row_ror:8), on the VALU
+__device__ __forceinline__ float xor8(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));
+}
 
 // one wave per (token, head): vec[t][h][d] = {w, a u, k, r}, un[t][h][d] = u
 __global__ __launch_bounds__(64) void delta_prep_kernel(DeltaArgs p, int T, float4* __restrict__ vec,
@@ -157,7 +161,7 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float
       float uS = 0.f;
 #pragma unroll
       for (int j = 0; j < DQ; ++j) uS = fmaf(xu[r][j], S[j], uS);
-      uS += __shfl_xor(uS, 8, 64);
+      uS += xor8(uS);
       uS += xor16(uS);
       uS += xor32(uS);
       float o = 0.f;
@@ -167,7 +171,7 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(DeltaArgs p, const float
         S[j] = fmaf(x.z, vv, fmaf(-x.y, uS, x.x * S[j]));
         o = fmaf(x.w, S[j], o);
       }
-      o += __shfl_xor(o, 8, 64);
+      o += xor8(o);
       o += xor16(o);
       o += xor32(o);
       if (con && q == 0) oraw[(int64_t)(tb + i) * p.H * D + h * D + c] = o;
