@@ -219,13 +219,18 @@ __device__ __forceinline__ bf16x8 frag16(const bf16_t* rowp, int k, int K, bool 
   return as_bf16x8(v);
 }
 
-__device__ __forceinline__ float group16_max(float v) {  // over the 16 lanes that share l >> 4
-  v = fmaxf(v, __shfl_xor(v, 8, 64)); v = fmaxf(v, __shfl_xor(v, 4, 64));
-  v = fmaxf(v, __shfl_xor(v, 2, 64)); v = fmaxf(v, __shfl_xor(v, 1, 64));
+// reductions over the 16 lanes that share l >> 4: rotations by 8, 4, 2, 1 inside the DPP row (VALU, no LDS)
+template <int CTRL>
+__device__ __forceinline__ float row_rot(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float group16_max(float v) {
+  v = fmaxf(v, row_rot<0x128>(v)); v = fmaxf(v, row_rot<0x124>(v));
+  v = fmaxf(v, row_rot<0x122>(v)); v = fmaxf(v, row_rot<0x121>(v));
   return v;
 }
 __device__ __forceinline__ float group16_sum(float v) {
-  v += __shfl_xor(v, 8, 64); v += __shfl_xor(v, 4, 64); v += __shfl_xor(v, 2, 64); v += __shfl_xor(v, 1, 64);
+  v += row_rot<0x128>(v); v += row_rot<0x124>(v); v += row_rot<0x122>(v); v += row_rot<0x121>(v);
   return v;
 }
 
