@@ -76,8 +76,8 @@ class HybridModel:
         self.tp = tp or TPGroup()
         if self.tp.size > 1:
             raise ValueError("layered hybrid models run on one GPU per replica (tensor_parallel_size 1)")
-        if quantization:
-            raise ValueError("layered hybrid models have no quantized path")
+        if (quantization or "none").lower() not in ("none", ""):
+            raise ValueError(f"layered hybrid models have no quantized path (quantization={quantization!r})")
         if dtype not in ("bfloat16", "float32"):
             raise ValueError(f"dtype {dtype!r}: bfloat16 or float32")
         self.f32 = dtype == "float32"
