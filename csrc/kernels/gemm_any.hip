@@ -47,6 +47,7 @@ __device__ __forceinline__ float epi_val(const AnyGemmArgs& p, float g, float u)
     return gg * sigmoidf_(p.alpha * gg) * (uu + 1.f);
   }
   if (p.act == 3) return tanhf(g);
+  if (p.act == 4) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
   return g;
 }
 

@@ -1,0 +1,190 @@
+// Linear attention with decay: one fp32 state matrix S [key][value] per (sequence, head) kept in a state
+// slot between steps,
+//   S <- diag(a_t) S + k_t v_t^T,   o_t = S^T (q_scale q_t)
+// with a_t either a constant per head or sigmoid(z_t)^(1 / tau) per key channel (z fp32), optionally
+// silu on q, k and v, then an RMS norm of o (per head, or over the concatenated heads) and an output
+// gate silu(g) or sigmoid(g). Key and value sizes may differ. Three launches:
+//   prep   (token, head) parallel: the fp32 per-channel triples {a, k, q_scale q} and the values.
+//   scan   the recurrence. Column v of S depends on no other column, so a head's value columns are split
+//          into slices of 8 and every (sequence, head, slice) is one wave: lane = (key group of eight,
+//          column), ceil(D / 8) state entries in registers; per token one FMA pair per entry and three
+//          lane exchanges for o. Tokens are staged through LDS, the next batch loaded into registers
+//          while the current one computes. A sequence's tokens of the step run in order from the slot's
+//          state; a portion that starts at position 0 starts from zero, so a reused slot needs no clearing.
+//   finish token parallel: norm, norm weight, output gate, store in the activation dtype.
+#include "common.h"
+#include "seq_launchers.h"
+
+namespace vgate {
+namespace {
+
+__device__ __forceinline__ float ldx(const void* p, int64_t i, int f32) {
+  return f32 ? reinterpret_cast<const float*>(p)[i] : bf2f(reinterpret_cast<const bf16_t*>(p)[i]);
+}
+__device__ __forceinline__ float sigm(float x) { return 1.f / (1.f + expf(-x)); }
+__device__ __forceinline__ float silu_f(float x) { return x * sigm(x); }
+// log(sigmoid(z)) without overflow on either side
+__device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+__device__ __forceinline__ float xor8(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));
+}
+
+// one workgroup per token: vec[t][h][d] = {a, k, q}, vals[t][h][c] = v
+__global__ __launch_bounds__(256) void linear_prep_kernel(LinearAttnArgs p, float4* __restrict__ vec,
+                                                           float* __restrict__ vals) {
+  const int t = blockIdx.x;
+  if (t >= p.query_start[p.S]) return;  // padding rows of a graph bucket
+  const int HD = p.H * p.D, HV = p.H * p.V;
+  const float inv_tau = 1.f / p.tau;
+  for (int e = threadIdx.x; e < HD; e += blockDim.x) {
+    float q = ldx(p.q, (int64_t)t * p.ldq + e, p.f32), k = ldx(p.k, (int64_t)t * p.ldk + e, p.f32);
+    if (p.in_silu) { q = silu_f(q); k = silu_f(k); }
+    const float a = p.z != nullptr ? expf(log_sigmoid(p.z[(int64_t)t * p.ldz + e]) * inv_tau) : p.head_decay[e / p.D];
+    vec[(int64_t)t * HD + e] = make_float4(a, k, q * p.q_scale, 0.f);
+  }
+  for (int e = threadIdx.x; e < HV; e += blockDim.x) {
+    const float v = ldx(p.v, (int64_t)t * p.ldv + e, p.f32);
+    vals[(int64_t)t * HV + e] = p.in_silu ? silu_f(v) : v;
+  }
+}
+
+// lane = 8 * q + c: key group q of 8 (keys [q dq, (q + 1) dq) with dq = ceil(D / 8) <= DQ), value column c0 + c
+template <int DQ, int TC>
+__global__ __launch_bounds__(64) void linear_scan_kernel(LinearAttnArgs p, const float4* __restrict__ vec,
+                                                          const float* __restrict__ vals, float* __restrict__ oraw) {
+  constexpr int QV = DQ + 1;             // padded group stride: the groups' broadcast reads hit different banks
+  constexpr int NE = (8 * DQ + 63) / 64;  // channels a lane stages per token
+  __shared__ float4 lv[2][TC][8 * QV];
+  __shared__ float lvv[2][TC][8];
+  const int s = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * 8;
+  const int slot = p.state_slots[s];
+  const int t0 = p.query_start[s], t1 = p.query_start[s + 1];
+  if (slot < 0 || t1 <= t0) return;
+  const int D = p.D, V = p.V, lane = threadIdx.x;
+  const int q = lane >> 3, c = c0 + (lane & 7);
+  const int dq = (D + 7) >> 3;
+  const int k0 = q * dq;
+  const bool con = c < V;
+  const int pos0 = p.context_lens[s] - (t1 - t0);
+  float* sp = p.state + ((int64_t)slot * p.H + h) * D * V;
+  float S[DQ];
+#pragma unroll
+  for (int j = 0; j < DQ; ++j)
+    S[j] = (con && j < dq && k0 + j < D && pos0 > 0) ? sp[(int64_t)(k0 + j) * V + c] : 0.f;
+  float4 pv[TC][NE];
+  float pvv[(TC * 8 + 63) / 64];
+  auto fetch = [&](int tb) {
+#pragma unroll
+    for (int i = 0; i < TC; ++i)
+#pragma unroll
+      for (int e = 0; e < NE; ++e) {
+        const int d = lane + 64 * e, t = tb + i;
+        const bool ok = d < D && t < t1;
+        pv[i][e] = ok ? vec[((int64_t)t * p.H + h) * D + d] : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    {  // TC x 8 values, lane -> (token, column)
+      const int t = tb + (lane >> 3), cc = c0 + (lane & 7);
+      pvv[0] = ((lane >> 3) < TC && t < t1 && cc < V) ? vals[((int64_t)t * p.H + h) * V + cc] : 0.f;
+    }
+  };
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < TC; ++i)
+#pragma unroll
+      for (int e = 0; e < NE; ++e) {
+        const int d = lane + 64 * e;
+        if (d < D) lv[buf][i][(d / dq) * QV + (d % dq)] = pv[i][e];
+      }
+    if ((lane >> 3) < TC) lvv[buf][lane >> 3][lane & 7] = pvv[0];
+  };
+  // entries of channels past D are zeroed once and never written: the token loops run DQ iterations with
+  // no bounds test (a = k = q = 0 leaves S and o alone)
+  for (int e = lane; e < 2 * TC * 8 * QV; e += 64) (&lv[0][0][0])[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+  __syncthreads();
+  fetch(t0);
+  put(0);
+  __syncthreads();
+  int buf = 0;
+  for (int tb = t0; tb < t1; tb += TC) {
+    const bool more = tb + TC < t1;
+    if (more) fetch(tb + TC);
+    const int nt = min(TC, t1 - tb);
+#pragma unroll
+    for (int i = 0; i < TC; ++i) {
+      if (i >= nt) break;
+      const float4* tv = &lv[buf][i][q * QV];
+      const float vv = lvv[buf][i][lane & 7];
+      float o = 0.f;
+#pragma unroll
+      for (int j = 0; j < DQ; ++j) {
+        const float4 x = tv[j];  // {a, k, q}
+        S[j] = fmaf(x.y, vv, x.x * S[j]);
+        o = fmaf(x.z, S[j], o);
+      }
+      o += xor8(o);
+      o += xor16(o);
+      o += xor32(o);
+      if (con && q == 0) oraw[((int64_t)(tb + i) * p.H + h) * V + c] = o;
+    }
+    if (more) {
+      put(buf ^ 1);
+      __syncthreads();
+      buf ^= 1;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < DQ; ++j)
+    if (con && j < dq && k0 + j < D) sp[(int64_t)(k0 + j) * V + c] = S[j];
+}
+
+// one workgroup per token; waves take heads in turn
+__global__ __launch_bounds__(256) void linear_finish_kernel(LinearAttnArgs p, const float* __restrict__ oraw) {
+  __shared__ float red[16];
+  const int t = blockIdx.x;
+  if (t >= p.query_start[p.S]) return;
+  const int H = p.H, V = p.V, HV = H * V;
+  const float* o = oraw + (int64_t)t * HV;
+  auto emit = [&](int e, float y) {
+    const float g = ldx(p.g, (int64_t)t * p.ldg + e, p.f32);
+    y *= p.gate_silu ? silu_f(g) : sigm(g);
+    const int64_t oi = (int64_t)t * p.ldo + e;
+    if (p.f32) reinterpret_cast<float*>(p.out)[oi] = y;
+    else reinterpret_cast<bf16_t*>(p.out)[oi] = f2bf(y);
+  };
+  if (p.norm_all) {
+    float ss = 0.f;
+    for (int e = threadIdx.x; e < HV; e += blockDim.x) ss = fmaf(o[e], o[e], ss);
+    ss = block_reduce_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float)HV + p.eps);
+    for (int e = threadIdx.x; e < HV; e += blockDim.x) emit(e, o[e] * inv * p.nw[e]);
+    return;
+  }
+  const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int h = wv; h < H; h += 4) {
+    float ss = 0.f;
+    for (int c = lane; c < V; c += 64) ss = fmaf(o[h * V + c], o[h * V + c], ss);
+    ss = wave_reduce_sum(ss);
+    const float inv = 1.f / sqrtf(ss / (float)V + p.eps);
+    for (int c = lane; c < V; c += 64) emit(h * V + c, o[h * V + c] * inv * p.nw[c]);
+  }
+}
+
+}  // namespace
+
+// scratch: T * H * (4 D + 2 V) floats ({a, k, q, -} per key channel, the values, the raw outputs)
+void launch_linear_attn(const LinearAttnArgs& a, int T, float* scratch, hipStream_t st) {
+  if (a.S <= 0 || a.H <= 0 || T <= 0) return;
+  const int64_t nk = (int64_t)T * a.H * a.D, nv = (int64_t)T * a.H * a.V;
+  float4* vec = reinterpret_cast<float4*>(scratch);
+  float* vals = scratch + 4 * nk;
+  float* oraw = vals + nv;
+  hipLaunchKernelGGL(linear_prep_kernel, dim3(T), dim3(256), 0, st, a, vec, vals);
+  const dim3 grid(a.S, a.H, (a.V + 7) / 8);
+  if (a.D <= 32) hipLaunchKernelGGL((linear_scan_kernel<4, 8>), grid, dim3(64), 0, st, a, vec, vals, oraw);
+  else if (a.D <= 64) hipLaunchKernelGGL((linear_scan_kernel<8, 8>), grid, dim3(64), 0, st, a, vec, vals, oraw);
+  else if (a.D <= 128) hipLaunchKernelGGL((linear_scan_kernel<16, 8>), grid, dim3(64), 0, st, a, vec, vals, oraw);
+  else hipLaunchKernelGGL((linear_scan_kernel<32, 4>), grid, dim3(64), 0, st, a, vec, vals, oraw);
+  hipLaunchKernelGGL(linear_finish_kernel, dim3(T), dim3(256), 0, st, a, oraw);
+}
+
+}  // namespace vgate

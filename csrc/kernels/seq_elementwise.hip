@@ -73,6 +73,40 @@ __global__ __launch_bounds__(256) void gated_residual_kernel(float* __restrict__
   }
 }
 
+__global__ __launch_bounds__(256) void cast_rows_kernel(const float* __restrict__ x, bf16_t* __restrict__ y, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) y[i] = f2bf(x[i]);
+}
+
+// one workgroup per token; every element is read and written by the same thread, so out may be x and
+// mix may be x
+__global__ __launch_bounds__(256) void post_norm_add_kernel(PostNormArgs a) {
+  __shared__ float red[16];
+  const int t = blockIdx.x;
+  const int64_t ro = (int64_t)t * a.W;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < a.W; c += blockDim.x) {
+    float u = a.s1 * ldx(a.y1, ro + c, a.y_f32);
+    if (a.y2 != nullptr) u = fmaf(a.s2, ldx(a.y2, ro + c, a.y_f32), u);
+    ss = fmaf(u, u, ss);
+  }
+  ss = block_reduce_sum(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)a.W + a.eps);
+  for (int c = threadIdx.x; c < a.W; c += blockDim.x) {
+    float u = a.s1 * ldx(a.y1, ro + c, a.y_f32);
+    if (a.y2 != nullptr) u = fmaf(a.s2, ldx(a.y2, ro + c, a.y_f32), u);
+    float r = a.x[ro + c] + u * inv * a.w[c];
+    a.out[ro + c] = r;
+    if (a.hist != nullptr) {   // depth average, planes ascending; the last plane is the row just made
+      float m = 0.f;
+      for (int j = 0; j + 1 < a.planes; ++j) m = fmaf(a.coef[j], a.hist[(int64_t)j * a.hist_ps + ro + c], m);
+      r = fmaf(a.coef[a.planes - 1], r, m);
+      a.mix[ro + c] = r;
+    }
+    if (a.act_out != nullptr) reinterpret_cast<bf16_t*>(a.act_out)[ro + c] = f2bf(r);
+  }
+}
+
 // one thread per token: `top` rounds of arg-max over the corrected scores (lowest index wins a tie)
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ z, const float* __restrict__ corr,
                                                         int T, int E, int top, float norm_eps,
@@ -140,6 +174,18 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const void* __restrict
 }
 
 }  // namespace
+
+void launch_cast_rows(const float* x, void* y, int T, int n, hipStream_t st) {
+  const int64_t tot = (int64_t)T * n;
+  if (tot <= 0) return;
+  hipLaunchKernelGGL(cast_rows_kernel, dim3((unsigned)((tot + 255) / 256)), dim3(256), 0, st, x,
+                     reinterpret_cast<bf16_t*>(y), tot);
+}
+
+void launch_post_norm_add(const PostNormArgs& a, hipStream_t st) {
+  if (a.T <= 0 || a.W <= 0) return;
+  hipLaunchKernelGGL(post_norm_add_kernel, dim3(a.T), dim3(256), 0, st, a);
+}
 
 void launch_norm_rows(const void* x, int64_t ldx_, int x_f32, const int32_t* rows, const float* w, int w_scalar,
                       float eps, void* y, int64_t ldy, int y_f32, int M, int n, hipStream_t st) {

@@ -1,7 +1,9 @@
 // Host-side launcher declarations for the kernels of layered hybrid models: row-major GEMMs of any
 // shape (batched per head, grouped per expert, gated-linear-unit pairs), row norms with a scalar or a
 // vector weight over an fp32 residual stream, latent (compressed key/value) attention over a paged
-// cache, the generalized delta rule over per-sequence state slots, and mixture-of-experts routing.
+// cache, sliding-window attention with pooled blocks and sinks over paged key / value caches, the
+// generalized delta rule and decayed linear attention over per-sequence state slots, the post-norm
+// residual update with depth averaging, and mixture-of-experts routing.
 // Activations are bf16 or fp32 (`f32` flags); the residual stream, scores, norms and states are fp32.
 #pragma once
 #include <hip/hip_runtime.h>
@@ -22,7 +24,8 @@ struct AnyGemmArgs {
   const int32_t* group_off = nullptr;   // [groups + 1] row ranges (device): rows of group g use W + g * w_bs
   int groups = 0;
   int act = 0;                          // 0 none; 1 silu(g) * u; 2 clamped: g' = min(g, L), u' = clamp(u, -L, L),
-  float limit = 0.f;                    //   g' * sigmoid(alpha g') * (u' + 1); 3 tanh (single matrix)
+  float limit = 0.f;                    //   g' * sigmoid(alpha g') * (u' + 1); 3 tanh (single matrix);
+                                        //   4 gelu_tanh(g) * u
   float alpha = 1.702f;
   int in_f32 = 0, out_f32 = 0, gate_f32 = 0;
 };
@@ -37,6 +40,23 @@ void launch_embed_rows(const int32_t* ids, const int32_t* prev, const void* tabl
 // x += y1 * sigmoid(g1 + b1) [+ y2 * sigmoid(g2 + b2)]; null g: plain add
 void launch_gated_residual(float* x, const void* y1, const void* g1, int64_t ldg1, const float* b1, const void* y2,
                            const void* g2, int64_t ldg2, const float* b2, int f32, int T, int W, hipStream_t st);
+
+// y = x rounded to the activation dtype (bf16), rows of n
+void launch_cast_rows(const float* x, void* y, int T, int n, hipStream_t st);
+// out = x + u * rsqrt(mean(u^2) + eps) * w, u = s1 y1 [+ s2 y2] (fp32; out may alias x). With hist
+// ([planes][T][W] fp32, plane stride hist_ps, whose last used plane is out): mix = sum_j coef[j] hist[j].
+// act_out (bf16): a copy of mix, or of out without hist.
+struct PostNormArgs {
+  const float* x = nullptr; const void* y1 = nullptr; const void* y2 = nullptr; int y_f32 = 0;
+  float s1 = 1.f, s2 = 1.f, eps = 0.f;
+  const float* w = nullptr;
+  float* out = nullptr;
+  const float* hist = nullptr; int64_t hist_ps = 0; int planes = 0; const float* coef = nullptr;
+  float* mix = nullptr;
+  void* act_out = nullptr;
+  int T = 0, W = 0;
+};
+void launch_post_norm_add(const PostNormArgs& a, hipStream_t st);
 
 struct LatentArgs {
   int rank = 0, rot = 0, rot_dims = 0;  // latent size, rotated key size, leading rotated dims (<= rot, even)
@@ -72,6 +92,49 @@ struct DeltaArgs {
 };
 // T rows; scratch: T * H * D * 6 floats (the prepared per-channel vectors and the raw outputs)
 void launch_delta_rule(const DeltaArgs& a, int T, float* scratch, hipStream_t st);
+
+// Sliding-window attention over paged key / value caches with optional pooled blocks (window_attn.hip).
+struct WindowArgs {
+  int H = 0, G = 0, D = 0, V = 0;       // query heads, key/value heads, key size, value size
+  int page = 0, npool = 0;              // tokens per page; pooled rows per page (0: no pooled caches)
+  int rot_dims = 0, window = 0, pool = 0;
+  int f32 = 0, T = 0, S = 0, max_blocks = 0;
+  const float* inv_freq = nullptr;      // [rot_dims / 2]
+  const float* v_freq = nullptr;        // [V / 2]: values are turned by their position (null: not)
+  const float* sink = nullptr;          // [H] logits that only enter the softmax denominator (null: none)
+  const int32_t* positions = nullptr;   // [T]
+  const int32_t* slots = nullptr;       // [T] page * tokens-per-page + offset of each token (-1: padding)
+  const int32_t* block_tables = nullptr; const int32_t* context_lens = nullptr; const int32_t* query_start = nullptr;
+  void* kc = nullptr; void* vc = nullptr;  // [pages][G][page][D | V]
+  void* kp = nullptr; void* vp = nullptr;  // [pages][G][npool][D | V]
+};
+size_t window_attn_lds_bytes(const WindowArgs& a, int heads_per_block);
+bool window_attn_fits(const WindowArgs& a);   // sizes the kernels' LDS and register budgets take
+// q / k norm (qw, kw null: none; norm_all: one norm over the whole projection) + rotation + paged stores; q_out [T][H * D]
+void launch_window_write(const WindowArgs& a, const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
+                         int64_t ldv, const float* qw, const float* kw, float eps, int norm_all, void* q_out,
+                         hipStream_t st);
+// pooled rows of the blocks this step's tokens complete
+void launch_window_pool(const WindowArgs& a, hipStream_t st);
+// out[t][h][:V] = softmax over (pooled blocks before the window, window tokens [, sink]) of scale q . key, times values
+void launch_window_attn(const WindowArgs& a, const void* q, float scale, void* out, hipStream_t st);
+
+// Linear attention with decay over per-sequence state slots (linear_attn.hip).
+struct LinearAttnArgs {
+  const void* q = nullptr; const void* k = nullptr; const void* v = nullptr; const void* g = nullptr;
+  int64_t ldq = 0, ldk = 0, ldv = 0, ldg = 0;   // activation dtype rows: q, k [H * D]; v, g [H * V]
+  const float* z = nullptr; int64_t ldz = 0;    // decay logits per key channel (null: head_decay)
+  const float* head_decay = nullptr;            // [H]
+  float tau = 1.f, q_scale = 1.f, eps = 0.f;
+  int in_silu = 0, norm_all = 0, gate_silu = 0;
+  const float* nw = nullptr;                    // [V], or [H * V] with norm_all
+  float* state = nullptr;                       // [slots][H][D][V]
+  const int32_t* state_slots = nullptr; const int32_t* context_lens = nullptr; const int32_t* query_start = nullptr;
+  void* out = nullptr; int64_t ldo = 0;
+  int S = 0, H = 0, D = 0, V = 0, f32 = 0;
+};
+// T rows; scratch: T * H * (4 D + 2 V) floats, 16-B aligned
+void launch_linear_attn(const LinearAttnArgs& a, int T, float* scratch, hipStream_t st);
 
 // idx, wts [T][top]: the `top` largest of sigmoid(z) + corr; wts = sigmoid(z) of the chosen / their sum
 void launch_moe_route(const float* z, const float* corr, int T, int E, int top, float norm_eps, int32_t* idx,

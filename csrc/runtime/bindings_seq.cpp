@@ -66,9 +66,9 @@ void gemm_any(const Tensor& a, const Tensor& w, Tensor& out, const OptT& w2, con
     TORCH_CHECK(act_f32(*w2, "w2") == g.in_f32 && w2->sizes() == w.sizes() && w2->strides() == w.strides(),
                 "gemm_any: w2 must match w");
     g.w2 = w2->data_ptr();
-    TORCH_CHECK(act == 1 || act == 2, "gemm_any: a weight pair needs act 1 or 2");
+    TORCH_CHECK(act == 1 || act == 2 || act == 4, "gemm_any: a weight pair needs act 1, 2 or 4");
   } else {
-    TORCH_CHECK(act == 0 || act == 3, "gemm_any: act 1 / 2 need a weight pair");
+    TORCH_CHECK(act == 0 || act == 3, "gemm_any: act 1 / 2 / 4 need a weight pair");
   }
   g.bias = f32p(bias, "bias", g.N);
   TORCH_CHECK(!(g.bias && B > 1), "gemm_any: bias only without batch");
@@ -252,6 +252,185 @@ void delta_rule(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor&
   vgate::launch_delta_rule(p, (int)T, scratch.data_ptr<float>(), cur_stream());
 }
 
+
+void cast_rows(const Tensor& x, Tensor& y) {
+  TORCH_CHECK(x.is_cuda() && x.scalar_type() == torch::kFloat32 && x.is_contiguous() && x.dim() == 2, "cast_rows: x fp32 [T, n]");
+  TORCH_CHECK(y.is_cuda() && y.scalar_type() == torch::kBFloat16 && y.is_contiguous() && y.dim() == 2 &&
+              y.size(1) == x.size(1) && y.size(0) <= x.size(0), "cast_rows: y bf16 [<= T, n]");
+  c10::DeviceGuard guard(x.device());
+  vgate::launch_cast_rows(x.data_ptr<float>(), y.data_ptr(), (int)y.size(0), (int)y.size(1), cur_stream());
+}
+
+void post_norm_add(const Tensor& x, const Tensor& y1, const Tensor& w, double eps, Tensor& out, double s1, const OptT& y2,
+                   double s2, const OptT& act_out, const OptT& hist, int64_t planes, const OptT& coef, const OptT& mix) {
+  auto f32_2d = [](const Tensor& t, const char* name) {
+    TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kFloat32 && t.is_contiguous() && t.dim() == 2, name, ": fp32 [T, W]");
+  };
+  f32_2d(x, "x"); f32_2d(out, "out");
+  vgate::PostNormArgs a;
+  a.T = (int)out.size(0); a.W = (int)out.size(1);
+  TORCH_CHECK(x.size(0) >= a.T && x.size(1) == a.W, "post_norm_add: x rows / width");
+  a.y_f32 = act_f32(y1, "y1");
+  TORCH_CHECK(y1.dim() == 2 && y1.is_contiguous() && y1.size(0) >= a.T && y1.size(1) == a.W, "post_norm_add: y1 [T, W]");
+  if (has(y2)) {
+    TORCH_CHECK(act_f32(*y2, "y2") == a.y_f32 && y2->dim() == 2 && y2->is_contiguous() && y2->size(0) >= a.T &&
+                y2->size(1) == a.W, "post_norm_add: y2 like y1");
+    a.y2 = y2->data_ptr();
+  }
+  OptT wo(w);
+  a.x = x.data_ptr<float>(); a.y1 = y1.data_ptr(); a.w = f32p(wo, "w", a.W); a.out = out.data_ptr<float>();
+  a.s1 = (float)s1; a.s2 = (float)s2; a.eps = (float)eps;
+  if (has(hist)) {
+    TORCH_CHECK(hist->is_cuda() && hist->scalar_type() == torch::kFloat32 && hist->dim() == 3 && hist->is_contiguous() &&
+                hist->size(2) == a.W && hist->size(1) >= a.T, "post_norm_add: hist fp32 [n, T, W]");
+    TORCH_CHECK(planes >= 1 && planes <= hist->size(0), "post_norm_add: planes");
+    TORCH_CHECK(out.data_ptr<float>() == hist->data_ptr<float>() + (planes - 1) * hist->stride(0),
+                "post_norm_add: out must be hist's plane planes - 1");
+    TORCH_CHECK(has(mix) && has(coef), "post_norm_add: hist needs coef and mix");
+    f32_2d(*mix, "mix");
+    TORCH_CHECK(mix->size(0) >= a.T && mix->size(1) == a.W, "post_norm_add: mix rows / width");
+    a.hist = hist->data_ptr<float>(); a.hist_ps = hist->stride(0); a.planes = (int)planes;
+    a.coef = f32p(coef, "coef", planes); a.mix = mix->data_ptr<float>();
+  }
+  if (has(act_out)) {
+    TORCH_CHECK(act_out->is_cuda() && act_out->scalar_type() == torch::kBFloat16 && act_out->is_contiguous() &&
+                act_out->dim() == 2 && act_out->size(0) >= a.T && act_out->size(1) == a.W, "post_norm_add: act_out bf16 [T, W]");
+    a.act_out = act_out->data_ptr();
+  }
+  c10::DeviceGuard guard(x.device());
+  vgate::launch_post_norm_add(a, cur_stream());
+}
+
+// caches kc [pages, G, page, D], vc [pages, G, page, V], pooled kp / vp [pages, G, npool, D | V]
+vgate::WindowArgs window_common(const Tensor& kc, const Tensor& vc, const OptT& kp, const OptT& vp, int64_t H, int64_t pool) {
+  vgate::WindowArgs a;
+  a.f32 = act_f32(kc, "kc");
+  TORCH_CHECK(kc.dim() == 4 && vc.dim() == 4 && kc.is_contiguous() && vc.is_contiguous() && act_f32(vc, "vc") == a.f32 &&
+              kc.size(0) == vc.size(0) && kc.size(1) == vc.size(1) && kc.size(2) == vc.size(2),
+              "window: kc [pages, G, page, D], vc [pages, G, page, V] of one dtype");
+  a.G = (int)kc.size(1); a.page = (int)kc.size(2); a.D = (int)kc.size(3); a.V = (int)vc.size(3); a.H = (int)H;
+  TORCH_CHECK(a.G >= 1 && H >= a.G && H % a.G == 0 && H + a.G <= 256, "window: heads a multiple of kv heads, at most 256 together");
+  a.kc = kc.data_ptr(); a.vc = vc.data_ptr();
+  a.pool = (int)pool;
+  TORCH_CHECK(pool >= 0, "window: pool");
+  if (pool > 0) {
+    TORCH_CHECK(has(kp) && has(vp), "window: pooled caches missing");
+    const int64_t np = (a.page + pool - 1) / pool;
+    for (const Tensor* t : {&*kp, &*vp})
+      TORCH_CHECK(t->dim() == 4 && t->is_contiguous() && act_f32(*t, "pooled cache") == a.f32 && t->size(0) == kc.size(0) &&
+                  t->size(1) == a.G && t->size(2) == np, "window: pooled caches [pages, G, ceil(page / pool), D | V]");
+    TORCH_CHECK(kp->size(3) == a.D && vp->size(3) == a.V, "window: pooled row widths");
+    a.npool = (int)np; a.kp = kp->data_ptr(); a.vp = vp->data_ptr();
+  }
+  TORCH_CHECK(vgate::window_attn_fits(a), "window: head sizes out of the kernels' range");
+  return a;
+}
+
+void window_write(const Tensor& q, const Tensor& k, const Tensor& v, const OptT& qw, const OptT& kw, double eps,
+                  bool norm_all, const Tensor& positions, const Tensor& slots, const Tensor& inv_freq, int64_t rot_dims,
+                  const OptT& v_freq, Tensor& kc, Tensor& vc, Tensor& q_out, int64_t H, int64_t G) {
+  auto a = window_common(kc, vc, c10::nullopt, c10::nullopt, H, 0);
+  TORCH_CHECK(G == a.G, "window_write: kv heads");
+  const int64_t T = q.size(0);
+  TORCH_CHECK(act_f32(q, "q") == a.f32 && act_f32(k, "k") == a.f32 && act_f32(v, "v") == a.f32 && q.dim() == 2 &&
+              k.dim() == 2 && v.dim() == 2 && k.size(0) == T && v.size(0) == T && q.size(1) == H * a.D &&
+              k.size(1) == G * a.D && v.size(1) == G * a.V, "window_write: q [T, H D], k [T, G D], v [T, G V] of the caches' dtype");
+  TORCH_CHECK(act_f32(q_out, "q_out") == a.f32 && q_out.is_contiguous() && q_out.dim() == 2 && q_out.size(0) == T &&
+              q_out.size(1) == H * a.D, "window_write: q_out [T, H D]");
+  TORCH_CHECK(rot_dims >= 0 && rot_dims <= a.D && rot_dims % 2 == 0, "window_write: rot_dims");
+  a.rot_dims = (int)rot_dims; a.T = (int)T;
+  OptT fo(inv_freq);
+  a.inv_freq = f32p(fo, "inv_freq", -1);
+  TORCH_CHECK(inv_freq.numel() >= rot_dims / 2, "window_write: inv_freq");
+  a.v_freq = f32p(v_freq, "v_freq", a.V / 2);
+  a.positions = i32p(positions, "positions", T);
+  a.slots = i32p(slots, "slots", T);  // values < pages * page: written from the step's block tables
+  TORCH_CHECK(has(qw) == has(kw), "window_write: q / k norm weights come together");
+  const float* qwp = f32p(qw, "qw", norm_all ? H * a.D : a.D);
+  const float* kwp = f32p(kw, "kw", norm_all ? G * a.D : a.D);
+  c10::DeviceGuard guard(q.device());
+  vgate::launch_window_write(a, q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), qwp, kwp,
+                             (float)eps, norm_all ? 1 : 0, q_out.data_ptr(), cur_stream());
+}
+
+void window_seq_meta(vgate::WindowArgs& a, const Tensor& block_tables, const Tensor& query_start) {
+  TORCH_CHECK(block_tables.dim() == 2, "window: block_tables [S, max_blocks]");
+  a.S = (int)block_tables.size(0); a.max_blocks = (int)block_tables.size(1);
+  a.block_tables = i32p(block_tables, "block_tables", 1);
+  a.query_start = i32p(query_start, "query_start", a.S + 1);  // values <= T: set by the step metadata
+}
+
+void window_pool(const Tensor& kc, const Tensor& vc, const OptT& kp, const OptT& vp, const Tensor& positions,
+                 const Tensor& block_tables, const Tensor& query_start, int64_t pool) {
+  TORCH_CHECK(pool >= 1, "window_pool: pool >= 1");
+  auto a = window_common(kc, vc, kp, vp, kc.size(1), pool);
+  window_seq_meta(a, block_tables, query_start);
+  a.T = (int)positions.numel();
+  a.positions = i32p(positions, "positions", a.T);
+  c10::DeviceGuard guard(kc.device());
+  vgate::launch_window_pool(a, cur_stream());
+}
+
+void window_attn(const Tensor& q, const Tensor& kc, const Tensor& vc, const OptT& kp, const OptT& vp,
+                 const Tensor& block_tables, const Tensor& context_lens, const Tensor& query_start, Tensor& out,
+                 double scale, int64_t H, int64_t window, int64_t pool, const OptT& sink, const OptT& v_freq) {
+  auto a = window_common(kc, vc, kp, vp, H, pool);
+  window_seq_meta(a, block_tables, query_start);
+  a.context_lens = i32p(context_lens, "context_lens", a.S);
+  const int64_t T = q.size(0);
+  TORCH_CHECK(act_f32(q, "q") == a.f32 && q.dim() == 2 && q.is_contiguous() && q.size(1) == H * a.D, "window_attn: q [T, H D]");
+  TORCH_CHECK(act_f32(out, "out") == a.f32 && out.dim() == 2 && out.is_contiguous() && out.size(0) == T &&
+              out.size(1) == H * a.V, "window_attn: out [T, H V]");
+  TORCH_CHECK(window >= 1, "window_attn: window >= 1");
+  a.T = (int)T; a.window = (int)window;
+  a.sink = f32p(sink, "sink", H);
+  a.v_freq = f32p(v_freq, "v_freq", a.V / 2);
+  c10::DeviceGuard guard(q.device());
+  vgate::launch_window_attn(a, q.data_ptr(), (float)scale, out.data_ptr(), cur_stream());
+}
+
+void linear_attn(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& g, const OptT& z, const OptT& head_decay,
+                 double tau, double q_scale, bool in_silu, const Tensor& nw, bool norm_all, bool gate_silu, Tensor& state,
+                 const Tensor& state_slots, const Tensor& context_lens, const Tensor& query_start, Tensor& out, double eps,
+                 Tensor& scratch) {
+  vgate::LinearAttnArgs p;
+  p.f32 = act_f32(q, "q");
+  TORCH_CHECK(state.is_cuda() && state.scalar_type() == torch::kFloat32 && state.is_contiguous() && state.dim() == 4,
+              "linear_attn: state fp32 [slots, H, D, V]");
+  p.H = (int)state.size(1); p.D = (int)state.size(2); p.V = (int)state.size(3);
+  TORCH_CHECK(p.D >= 1 && p.D <= 256 && p.V >= 1, "linear_attn: key size 1..256");
+  const int64_t T = q.size(0), HD = (int64_t)p.H * p.D, HV = (int64_t)p.H * p.V;
+  auto rows = [&](const Tensor& t, int64_t n, const char* name) {
+    TORCH_CHECK(act_f32(t, name) == p.f32 && t.dim() == 2 && t.size(0) == T && t.size(1) == n, "linear_attn: ", name, " [T, ", n, "]");
+  };
+  rows(q, HD, "q"); rows(k, HD, "k"); rows(v, HV, "v"); rows(g, HV, "g"); rows(out, HV, "out");
+  p.q = q.data_ptr(); p.k = k.data_ptr(); p.v = v.data_ptr(); p.g = g.data_ptr();
+  p.ldq = q.stride(0); p.ldk = k.stride(0); p.ldv = v.stride(0); p.ldg = g.stride(0);
+  p.out = out.data_ptr(); p.ldo = out.stride(0);
+  TORCH_CHECK(has(z) != has(head_decay), "linear_attn: either decay logits or one decay per head");
+  if (has(z)) {
+    TORCH_CHECK(z->is_cuda() && z->scalar_type() == torch::kFloat32 && z->dim() == 2 && z->stride(1) == 1 && z->size(0) == T &&
+                z->size(1) == HD, "linear_attn: z fp32 [T, H D]");
+    p.z = z->data_ptr<float>(); p.ldz = z->stride(0);
+    TORCH_CHECK(tau > 0, "linear_attn: tau > 0");
+  }
+  p.head_decay = f32p(head_decay, "head_decay", p.H);
+  OptT nwo(nw);
+  p.nw = f32p(nwo, "nw", norm_all ? HV : p.V);
+  p.tau = (float)tau; p.q_scale = (float)q_scale; p.eps = (float)eps;
+  p.in_silu = in_silu; p.norm_all = norm_all; p.gate_silu = gate_silu;
+  p.state = state.data_ptr<float>();
+  p.S = (int)state_slots.numel();
+  p.state_slots = i32p(state_slots, "state_slots", p.S);  // values < slots (or -1): set by the slot manager
+  p.context_lens = i32p(context_lens, "context_lens", p.S);
+  p.query_start = i32p(query_start, "query_start", p.S + 1);
+  TORCH_CHECK(scratch.is_cuda() && scratch.scalar_type() == torch::kFloat32 && scratch.is_contiguous() &&
+              scratch.numel() >= T * (4 * HD + 2 * HV), "linear_attn: scratch fp32 with T * H * (4 D + 2 V) elements");
+  TORCH_CHECK((reinterpret_cast<uintptr_t>(scratch.data_ptr()) & 15) == 0, "linear_attn: scratch must be 16-B aligned");
+  c10::DeviceGuard guard(q.device());
+  vgate::launch_linear_attn(p, (int)T, scratch.data_ptr<float>(), cur_stream());
+}
+
 void moe_route(const Tensor& z, const OptT& corr, int64_t top, double norm_eps, Tensor& idx, Tensor& wts) {
   TORCH_CHECK(z.is_cuda() && z.scalar_type() == torch::kFloat32 && z.is_contiguous() && z.dim() == 2, "moe_route: z fp32 [T, E]");
   const int64_t T = z.size(0), E = z.size(1);
@@ -312,6 +491,15 @@ void bind_seq(pybind11::module& m) {
         py::arg("cache"), py::arg("block_tables"), py::arg("context_lens"), py::arg("query_start"), py::arg("ol"),
         py::arg("scale"), py::arg("H"), py::arg("rank"), py::arg("rot"), py::arg("cache_t") = py::none());
   m.def("delta_rule", &delta_rule, "generalized delta rule recurrence over state slots + head norm + gate");
+  m.def("cast_rows", &cast_rows, "fp32 rows rounded to bf16");
+  m.def("post_norm_add", &post_norm_add, "out = x + rmsnorm(s1 y1 + s2 y2) * w, optional depth average and bf16 copy",
+        py::arg("x"), py::arg("y1"), py::arg("w"), py::arg("eps"), py::arg("out"), py::arg("s1") = 1.0,
+        py::arg("y2") = py::none(), py::arg("s2") = 1.0, py::arg("act_out") = py::none(), py::arg("hist") = py::none(),
+        py::arg("planes") = 0, py::arg("coef") = py::none(), py::arg("mix") = py::none());
+  m.def("window_write", &window_write, "q / k norm + rotation + paged key / value stores of window attention");
+  m.def("window_pool", &window_pool, "mean key / value rows of the blocks a step completes");
+  m.def("window_attn", &window_attn, "sliding-window attention with pooled blocks and an optional sink");
+  m.def("linear_attn", &linear_attn, "decayed linear attention recurrence over state slots + norm + gate");
   m.def("moe_route", &moe_route, "sigmoid router: corrected top-k choice, normalised uncorrected weights");
   m.def("moe_sort", &moe_sort, "counting sort of (token, choice) pairs by expert");
   m.def("moe_combine", &moe_combine, "weighted sum of a token's expert rows");

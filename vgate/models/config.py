@@ -8,6 +8,7 @@ name (random-init weights, used for benchmarks: there are no checkpoints here).
 from __future__ import annotations
 
 import json
+import math
 import os
 from dataclasses import asdict, dataclass, field, replace
 from pathlib import Path
@@ -142,6 +143,10 @@ class HybridArch:
     max_position: int = 1 << 20
     bos_token_id: int = 1
     eos_token_ids: tuple = (2,)
+    # how a layer combines its sublayers (a key of ``vgate.models.hybrid.ARRANGEMENTS``) and whether
+    # the stream that enters the next layer is a learned average of all earlier layers' results
+    arrangement: str = "gated_parallel"
+    depth_average: bool = False
 
     @property
     def num_layers(self) -> int:
@@ -158,10 +163,8 @@ class HybridArch:
         return i
 
     def num_params(self) -> int:
-        from vgate.models.mixers import layer_params
-        W = self.hidden_size
-        own = {self.owner(i) for i in range(len(self.layers))}
-        return 2 * self.vocab_size * W + 1 + sum(layer_params(self.layers[i], W) for i in sorted(own))
+        from vgate.models.hybrid import tensor_shapes
+        return sum(math.prod(shape) for shape in tensor_shapes(self).values())
 
     def to_dict(self) -> dict:
         return asdict(self)
@@ -184,8 +187,58 @@ def _zadirax_from_config(cfg: dict, name: str) -> HybridArch:
                       eos_token_ids=tuple(eos) if isinstance(eos, list) else (int(eos),))
 
 
+def _pozalorn_window(m: dict, qk_norm: str, rotate_values: bool, sink: bool, out_bias: bool) -> dict:
+    """Spec of a ``window_attention`` mixer from a Pozalorn attention block."""
+    mask = m["mask"]
+    return {"heads": int(m["heads"]), "kv_heads": int(m["kv_heads"]), "dim": int(m["dim"]), "vdim": int(m["vdim"]),
+            "scale": float(m["scale"]), "rot": dict(m["rot"]), "window": int(mask["size"]), "pool": int(mask.get("pool") or 0),
+            "qk_norm": qk_norm, "rotate_values": rotate_values, "sink": sink, "bias": True, "out_bias": out_bias}
+
+
+def _pozalorn_mixer(kind: str, m: dict) -> tuple:
+    """(key of ``vgate.models.mixers.MIXERS``, its spec) of a Pozalorn layer type. The choices the
+    design fixes (which norm, which activations, what is rotated) are written out here, so the mixers
+    themselves carry none of them."""
+    if kind == "gla":       # gated linear attention: per-channel decay sigmoid(z)^(1 / tau) from a low-rank gate
+        return "linear_attention", {"heads": int(m["heads"]), "dim": int(m["dim"]), "vdim": int(m["vdim"]),
+                                    "decay": {"kind": "channel", "tau": float(m["tau"])}, "q_scale": float(m["dim"]) ** -0.5,
+                                    "in_act": "none", "out_norm": "head", "gate_act": "silu"}
+    if kind == "attention":  # window + pooled blocks; whole-projection q / k norm; values rotated by their position
+        return "window_attention", _pozalorn_window(m, "all", True, False, False)
+    if kind == "parallel":   # sink-softmax window attention beside lightning attention (constant decay per head)
+        r = m["right"]
+        right = {"heads": int(r["heads"]), "dim": int(r["dim"]), "vdim": int(r["vdim"]),
+                 "decay": {"kind": "head", "values": [float(d) for d in r["decay"]]}, "q_scale": 1.0,
+                 "in_act": "silu", "out_norm": "all", "gate_act": "sigmoid"}
+        if len(right["decay"]["values"]) != right["heads"]:
+            raise ValueError("parallel.right: one decay per head")
+        return "parallel", {"left": ("window_attention", _pozalorn_window(m["left"], "head", False, True, True)),
+                            "right": ("linear_attention", right),
+                            "left_scale": float(m["left_scale"]), "right_scale": float(m["right_scale"])}
+    raise ValueError(f"Pozalorn has no layer type {kind!r}")
+
+
+def _pozalorn_from_config(cfg: dict, name: str) -> HybridArch:
+    """config.json of the Pozalorn design: sublayers read the stream itself, their outputs are normed
+    before they are added, and the next layer reads a learned average over all earlier results."""
+    layers = []
+    for L in cfg["layers"]:
+        kind, spec = _pozalorn_mixer(L["type"], L["mixer"])
+        mlp = dict(L["mlp"]) if L.get("mlp") else None
+        if mlp is not None:
+            if mlp.get("kind") != "dense":
+                raise ValueError(f"Pozalorn feed-forward kind {mlp.get('kind')!r}")
+            mlp["act"] = "gelu_tanh"
+        layers.append(LayerSpec(kind=kind, mixer=spec, mlp=mlp))
+    eos = cfg.get("eos_token_id", 2)
+    return HybridArch(name=name, family="pozalorn", hidden_size=int(cfg["width"]), vocab_size=int(cfg["vocab"]),
+                      layers=tuple(layers), rms_eps=float(cfg["norm"]["eps"]), bos_token_id=int(cfg.get("bos_token_id", 1)),
+                      eos_token_ids=tuple(eos) if isinstance(eos, list) else (int(eos),),
+                      arrangement="post_norm", depth_average=True)
+
+
 # config.json "architecture" -> parser of a layered hybrid design
-HYBRID_ARCHITECTURES = {"Zadirax": _zadirax_from_config}
+HYBRID_ARCHITECTURES = {"Zadirax": _zadirax_from_config, "Pozalorn": _pozalorn_from_config}
 
 
 def _zadirax_preset(name: str, width: int, vocab: int, pairs: int, heads: int, dim: int, ff: int, experts: int,

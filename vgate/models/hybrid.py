@@ -5,10 +5,15 @@ One forward pass = one engine step over a flat token batch (any mix of prompt po
 decoded tokens) with all step metadata in device buffers (:class:`vgate.runtime.step_meta.StepView`),
 as for the transformer families, so the same code is captured into a hipGraph per bucket.
 
-Layer (parallel arrangement, gated residual):
-    h  = x / sqrt(mean(x^2) + eps) * g            one scalar weight per norm; h in the activation dtype
-    P  = h @ [mixer inputs; rg1; rg2]^T           ONE fused input projection per layer
-    x += mixer(h) * sigmoid(P_rg1 + b1) + ff(h) * sigmoid(P_rg2 + b2)
+Layer arrangements (``ARRANGEMENTS``, chosen by ``HybridArch.arrangement``):
+  gated_parallel  h  = x / sqrt(mean(x^2) + eps) * g          one scalar weight per norm
+                  P  = h @ [mixer inputs; rg1; rg2]^T         ONE fused input projection per layer
+                  x += mixer(h) * sigmoid(P_rg1 + b1) + ff(h) * sigmoid(P_rg2 + b2)
+  post_norm       x += rmsnorm(mixer(x)) * w1;  x += rmsnorm(ff(x)) * w2
+                  (the sublayers read the stream itself, rounded to the activation dtype; their
+                  outputs are normed in fp32 before they are added)
+With ``HybridArch.depth_average`` the stream a layer hands on is a learned combination of the
+embedding output X_0 and every layer result X_1 .. X_(i+1): sum_j c_i[j] X_j (tensor ``l<i>.dwa``).
 A layer may run with another layer's weights (``weights_of``) while keeping its own cache or state.
 Activation dtype bf16 (MFMA GEMMs, fp32 accumulation) or fp32 (true fp32 FMA everywhere); the residual
 stream, norms, scores, routers and recurrent state are fp32 in both.
@@ -22,40 +27,63 @@ from pathlib import Path
 import torch
 
 from vgate.models.config import HybridArch
-from vgate.models.mixers import FEED_FORWARDS, MIXERS, Proj, _f32, _pad8, layer_shapes
+from vgate.models.mixers import FEED_FORWARDS, MIXERS, Proj, _f32, _pad8
 from vgate.ops import seq
 from vgate.parallel.comm import TPGroup
 
 
-class LayerWeights:
-    """The tensors of one weight-owning layer in kernel-ready form."""
+def _fuse_inputs(mixer, extra: list, width: int, device, f32: bool):
+    """Stack every matrix that multiplies the layer's input into ONE GEMM (segments padded to 8 rows,
+    the total to 64 columns). Returns (Proj, {name: (first column, columns)})."""
+    rows = list(mixer.in_rows) + extra
+    biases = dict(getattr(mixer, "in_bias", {}))
+    col, parts, bparts, off = {}, [], [], 0
+    for name, w in rows:
+        col[name] = (off, w.shape[0])
+        b = biases.get(name)
+        b = torch.zeros(w.shape[0], dtype=w.dtype) if b is None else b
+        w = _pad8(w)
+        parts.append(w)
+        bparts.append(torch.cat([b, torch.zeros(w.shape[0] - b.shape[0], dtype=b.dtype)]))
+        off += w.shape[0]
+    if off % 64:  # whole 64-column tiles: the widest alignment any of the GEMMs asks for
+        parts.append(torch.zeros(64 - off % 64, width, dtype=parts[0].dtype))
+        bparts.append(torch.zeros(64 - off % 64, dtype=bparts[0].dtype))
+    del mixer.in_rows
+    return Proj(torch.cat(parts), device, f32, bias=torch.cat(bparts) if biases else None), col
+
+
+class GatedParallelLayer:
+    """The tensors of one weight-owning layer of the ``gated_parallel`` arrangement in kernel-ready form."""
 
     def __init__(self, spec, width: int, eps: float, t: dict, device, f32: bool):
         mix = {k[4:]: v for k, v in t.items() if k.startswith("mix.")}
+        self.eps = eps
         self.mixer = MIXERS[spec.kind](spec.mixer, width, eps, mix, device, f32)
+        if spec.kind == "parallel":
+            raise ValueError("the gated_parallel arrangement takes single mixers")
         self.ff = None
         if spec.mlp:
             mlp = {k[4:]: v for k, v in t.items() if k.startswith("mlp.")}
             self.ff = FEED_FORWARDS[spec.mlp["kind"]](spec.mlp, width, mlp, device, f32)
         self.norm1 = _f32(t["norm1"].reshape(1), device)
-        rows = list(self.mixer.in_rows) + [("rg1", t["rg1"])]
+        extra = [("rg1", t["rg1"])]
         self.rg1_b = _f32(t["rg1.b"], device)
         self.rg2_b = None
         if self.ff is not None:
-            rows.append(("rg2", t["rg2"]))
+            extra.append(("rg2", t["rg2"]))
             self.rg2_b = _f32(t["rg2.b"], device)
-        self.col = {}
-        off = 0
-        parts = []
-        for name, w in rows:
-            self.col[name] = (off, w.shape[0])
-            w = _pad8(w)
-            parts.append(w)
-            off += w.shape[0]
-        if off % 64:  # whole 64-column tiles: the widest alignment any of the GEMMs asks for
-            parts.append(torch.zeros(64 - off % 64, width, dtype=parts[0].dtype))
-        self.proj = Proj(torch.cat(parts), device, f32)
-        del self.mixer.in_rows
+        self.proj, self.col = _fuse_inputs(self.mixer, extra, width, device, f32)
+
+    @staticmethod
+    def shapes(spec, width: int) -> dict:
+        out = {"norm1": ()}
+        out.update({"mix." + k: v for k, v in MIXERS[spec.kind].shapes(spec.mixer, width).items()})
+        out.update({"rg1": (width, width), "rg1.b": (width,)})
+        if spec.mlp:
+            out.update({"mlp." + k: v for k, v in FEED_FORWARDS[spec.mlp["kind"]].shapes(spec.mlp, width).items()})
+            out.update({"rg2": (width, width), "rg2.b": (width,)})
+        return out
 
     def cols(self, P: torch.Tensor, name: str) -> torch.Tensor:
         a, n = self.col[name]
@@ -63,6 +91,102 @@ class LayerWeights:
 
     def nbytes(self) -> int:
         return self.proj.nbytes() + self.mixer.nbytes() + (self.ff.nbytes() if self.ff else 0)
+
+    def run(self, st, sv, cache) -> None:
+        x, h = st.x, st.h
+        seq.norm_rows(x, self.norm1, self.eps, h, scalar=True)
+        P = self.proj(h)
+        y1 = self.mixer.forward(h, P, self.cols, sv, cache)
+        y2 = self.ff.forward(h) if self.ff is not None else None
+        seq.gated_residual(x, y1, self.cols(P, "rg1"), self.rg1_b, y2, self.cols(P, "rg2") if y2 is not None else None,
+                           self.rg2_b)
+
+
+class PostNormLayer:
+    """``post_norm`` arrangement: the mixer and the feed-forward read the stream itself; each output is
+    RMS-normed (vector weight, fp32) and then added. The residual kernel also hands on the activation-
+    dtype copy the next GEMM reads and, for the layer's last sublayer, the depth average."""
+
+    def __init__(self, spec, width: int, eps: float, t: dict, device, f32: bool):
+        mix = {k[4:]: v for k, v in t.items() if k.startswith("mix.")}
+        self.eps = eps
+        self.mixer = MIXERS[spec.kind](spec.mixer, width, eps, mix, device, f32)
+        self.norm1 = _f32(t["norm1"], device)
+        self.ff = self.norm2 = None
+        if spec.mlp:
+            mlp = {k[4:]: v for k, v in t.items() if k.startswith("mlp.")}
+            self.ff = FEED_FORWARDS[spec.mlp["kind"]](spec.mlp, width, mlp, device, f32)
+            self.norm2 = _f32(t["norm2"], device)
+        self.dwa = _f32(t["dwa"], device) if "dwa" in t else None
+        self.proj, self.col = _fuse_inputs(self.mixer, [], width, device, f32)
+
+    @staticmethod
+    def shapes(spec, width: int) -> dict:
+        out = {"norm1": (width,)}
+        out.update({"mix." + k: v for k, v in MIXERS[spec.kind].shapes(spec.mixer, width).items()})
+        if spec.mlp:
+            out.update({"mlp." + k: v for k, v in FEED_FORWARDS[spec.mlp["kind"]].shapes(spec.mlp, width).items()})
+            out["norm2"] = (width,)
+        return out
+
+    def cols(self, P: torch.Tensor, name: str) -> torch.Tensor:
+        a, n = self.col[name]
+        return P[:, a: a + n]
+
+    def nbytes(self) -> int:
+        return self.proj.nbytes() + self.mixer.nbytes() + (self.ff.nbytes() if self.ff else 0)
+
+    def run(self, st, sv, cache) -> None:
+        """st.x: the stream entering the layer (fp32), st.h its activation-dtype copy; the layer's result
+        goes to st.result (plane i + 1 of the history when the model averages over depth) and what the
+        next layer reads replaces st.x / st.h."""
+        P = self.proj(st.h)
+        y = self.mixer.forward(st.h, P, self.cols, sv, cache)
+        y1, s1, y2, s2 = y if isinstance(y, tuple) else (y, 1.0, None, 1.0)
+        last = self.ff is None
+        seq.post_norm_add(st.x, y1, self.norm1, self.eps, st.result, s1=s1, y2=y2, s2=s2, **st.hand_on(last))
+        if not last:
+            yf = self.ff.forward(st.result if st.f32 else st.h, out_f32=True)
+            seq.post_norm_add(st.result, yf, self.norm2, self.eps, st.result, **st.hand_on(True))
+
+
+ARRANGEMENTS = {"gated_parallel": GatedParallelLayer, "post_norm": PostNormLayer}
+
+
+class _Stream:
+    """The residual stream of one step: ``x`` fp32 [T, W] and ``h``, its copy in the activation dtype
+    (``x`` itself in an fp32 model). With depth averaging ``hist`` [layers + 1, T, W] keeps the
+    embedding output and every layer's result, and ``x`` is the average the next layer reads."""
+
+    def __init__(self, T: int, W: int, layers: int, act_dtype, device, depth_average: bool, normed_input: bool):
+        # an fp32 model whose sublayers read the stream itself needs no copy: h is x
+        self.f32 = act_dtype == torch.float32 and not normed_input
+        self.hist = torch.empty(layers + 1, T, W, dtype=torch.float32, device=device) if depth_average else None
+        self.x = self.hist[0] if depth_average else torch.empty(T, W, dtype=torch.float32, device=device)
+        self.h = self.x if self.f32 else torch.empty(T, W, dtype=act_dtype, device=device)
+        self.mix = torch.empty(T, W, dtype=torch.float32, device=device) if depth_average else None
+        self.result, self.layer, self.coef = self.x, 0, None
+
+    def begin(self, i: int, coef) -> None:
+        self.layer, self.coef = i, coef
+        self.result = self.hist[i + 1] if self.hist is not None else self.x
+
+    def hand_on(self, last: bool) -> dict:
+        """Extra outputs of a residual kernel: the activation-dtype copy of what the next GEMM reads and,
+        after the layer's last sublayer, the depth average (which then is what the copy is made of)."""
+        kw = {}
+        if last and self.hist is not None:
+            kw.update(hist=self.hist, planes=self.layer + 2, coef=self.coef, mix=self.mix)
+        if not self.f32:
+            kw["act_out"] = self.h
+        return kw
+
+    def end(self) -> None:
+        if self.hist is not None:
+            self.x = self.mix
+            if self.f32:
+                self.h = self.x
+        # (without depth averaging the result was written over x in place)
 
 
 class HybridModel:
@@ -86,19 +210,24 @@ class HybridModel:
         W = arch.hidden_size
         tensors = load_tensors(arch, weights_path) if weights_path else random_tensors(arch, seed)
         self.embed = tensors["embed"].to(self.device, self.act_dtype).contiguous()
-        owned: dict[int, LayerWeights] = {}
-        self.layers: list[LayerWeights] = []
+        layer_cls = ARRANGEMENTS[arch.arrangement]
+        owned: dict = {}
+        self.layers: list = []
         for i, spec in enumerate(arch.layers):
             j = arch.owner(i)
             if j not in owned:
                 pre = f"l{j}."
                 t = {k[len(pre):]: v for k, v in tensors.items() if k.startswith(pre)}
-                owned[j] = LayerWeights(arch.layers[j], W, arch.rms_eps, t, self.device, self.f32)
+                owned[j] = layer_cls(arch.layers[j], W, arch.rms_eps, t, self.device, self.f32)
             if MIXERS[spec.kind] is not type(owned[j].mixer):
                 raise ValueError(f"layer {i} shares weights with layer {j} of another mixer type")
             self.layers.append(owned[j])
         self._owned = owned
-        self.final_norm = _f32(tensors["final.norm"].reshape(1), self.device)
+        # depth-average coefficients belong to the position in the stack, not to the (possibly shared) weights
+        self.depth_coef = [_f32(tensors[f"l{i}.dwa"], self.device) for i in range(arch.num_layers)] \
+            if arch.depth_average else None
+        self.scalar_norm = arch.arrangement != "post_norm"   # one number per norm, or a weight vector
+        self.final_norm = _f32(tensors["final.norm"].reshape(-1), self.device)
         self.head = Proj(tensors["head"], self.device, self.f32)
         self.capture_layers: list | None = None  # set to [] to record the residual stream after every layer
         self.last_resid = None
@@ -110,18 +239,12 @@ class HybridModel:
 
     def cache_bytes_per_block(self, block_size: int) -> int:
         """Bytes one cache page costs over all layers with a paged cache."""
-        n = 0
-        for L in self.layers:
-            if L.mixer.cache == "paged":
-                s = L.mixer.cache_shape(1, block_size, 1)
-                n += math.prod(s) * torch.empty(0, dtype=L.mixer.cache_dtype()).element_size()
-        return max(n, 1)
+        return max(sum(L.mixer.page_bytes(block_size) for L in self.layers), 1)
 
     def allocate_caches(self, num_blocks: int, block_size: int, num_slots: int) -> list:
-        """One tensor per layer: a paged cache [blocks, page, row] or a state [slots, ...] (zeroed:
-        stale rows are always finite)."""
-        return [torch.zeros(L.mixer.cache_shape(num_blocks, block_size, num_slots), dtype=L.mixer.cache_dtype(),
-                            device=self.device) for L in self.layers]
+        """Per layer what its mixer keeps between steps: a paged cache, a state [slots, ...], or a tuple
+        of these (zeroed: stale rows are always finite)."""
+        return [L.mixer.allocate(num_blocks, block_size, num_slots, self.device) for L in self.layers]
 
     # ---------------------------------------------------------------- forward
     def forward(self, sv, caches, part_size: int = 0, return_hidden: bool = False) -> torch.Tensor:
@@ -130,18 +253,18 @@ class HybridModel:
         T = sv.T
         W = self.arch.hidden_size
         dev, eps = self.device, self.arch.rms_eps
-        x = torch.empty(T, W, dtype=torch.float32, device=dev)
-        seq.embed_rows(sv.ids, self.embed, x, prev=sv.prev_tokens)
-        h = torch.empty(T, W, dtype=self.act_dtype, device=dev)
+        st = _Stream(T, W, len(self.layers), self.act_dtype, dev, self.arch.depth_average,
+                     normed_input=self.arch.arrangement != "post_norm")
+        seq.embed_rows(sv.ids, self.embed, st.x, prev=sv.prev_tokens)
+        if self.arch.arrangement == "post_norm" and not self.f32:
+            seq.cast_rows(st.x, st.h)   # (the gated_parallel arrangement makes h with its norm)
         for li, L in enumerate(self.layers):
-            seq.norm_rows(x, L.norm1, eps, h, scalar=True)
-            P = L.proj(h)
-            y1 = L.mixer.forward(h, P, L.cols, sv, caches[li])
-            y2 = L.ff.forward(h) if L.ff is not None else None
-            seq.gated_residual(x, y1, L.cols(P, "rg1"), L.rg1_b, y2, L.cols(P, "rg2") if y2 is not None else None,
-                               L.rg2_b)
+            st.begin(li, self.depth_coef[li] if self.depth_coef else None)
+            L.run(st, sv, caches[li])
+            st.end()
             if self.capture_layers is not None:
-                self.capture_layers.append(x.clone())
+                self.capture_layers.append(st.x.clone())
+        x = st.x
         self.last_resid = x
         if return_hidden:
             return x
@@ -156,18 +279,22 @@ class HybridModel:
     def logits_of(self, x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         """fp32 logits [len(rows), vocab] of rows of the residual stream (final norm + head)."""
         hn = torch.empty(rows.numel(), x.shape[1], dtype=self.act_dtype, device=x.device)
-        seq.norm_rows(x, self.final_norm, self.arch.rms_eps, hn, rows=rows, scalar=True)
+        seq.norm_rows(x, self.final_norm, self.arch.rms_eps, hn, rows=rows, scalar=self.scalar_norm)
         return self.head(hn, out_f32=True, out=out)[:, : self.arch.vocab_size]
 
 
 # ------------------------------------------------------------------------------------------ weights
-def tensor_shapes(arch: HybridArch) -> dict:
-    """name -> shape of every tensor of a checkpoint of ``arch`` (weight-owning layers only)."""
+def tensor_shapes(arch: HybridArch, nominal: int | None = 16) -> dict:
+    """name -> shape of every tensor of a checkpoint of ``arch`` (weight-owning layers only). A size
+    that only a checkpoint's tensors give (a low-rank gate's width) is ``nominal``; None leaves it open."""
     W = arch.hidden_size
-    out = {"embed": (arch.vocab_size, W), "final.norm": (), "head": (arch.vocab_size, W)}
+    vector = arch.arrangement == "post_norm"
+    out = {"embed": (arch.vocab_size, W), "final.norm": (W,) if vector else (), "head": (arch.vocab_size, W)}
     for i in sorted({arch.owner(i) for i in range(arch.num_layers)}):
-        out.update({f"l{i}.{k}": v for k, v in layer_shapes(arch.layers[i], W).items()})
-    return out
+        out.update({f"l{i}.{k}": v for k, v in ARRANGEMENTS[arch.arrangement].shapes(arch.layers[i], W).items()})
+    if arch.depth_average:
+        out.update({f"l{i}.dwa": (i + 2,) for i in range(arch.num_layers)})
+    return {k: tuple(nominal if d is None else d for d in v) for k, v in out.items()}
 
 
 def load_tensors(arch: HybridArch, path: str) -> dict:
@@ -184,14 +311,12 @@ def load_tensors(arch: HybridArch, path: str) -> dict:
         with safe_open(str(f), framework="pt", device="cpu") as h:
             for k in h.keys():
                 t[k] = h.get_tensor(k)
-    for name, shape in tensor_shapes(arch).items():
+    for name, shape in tensor_shapes(arch, nominal=None).items():
         if name not in t:
             raise KeyError(f"checkpoint lacks tensor {name}")
         got = tuple(t[name].shape)
-        if name.endswith("mix.w1"):
-            ok = len(got) == 2 and got[1] == shape[1]
-        elif name.endswith("mix.w2"):
-            ok = len(got) == 2 and got[0] == shape[0] and got[1] == t[name[:-1] + "1"].shape[0]
+        if None in shape:   # a size only the tensors give (the mixer checks that its tensors agree on it)
+            ok = len(got) == len(shape) and all(w is None or g == w for g, w in zip(got, shape))
         else:
             ok = got == tuple(shape) or (math.prod(got) == 1 and math.prod(shape) == 1)
         if not ok:
@@ -206,10 +331,13 @@ def random_tensors(arch: HybridArch, seed: int = 0) -> dict:
     out = {}
     for name, shape in tensor_shapes(arch).items():
         leaf = name.split(".")[-1] if not name.endswith(".b") else "b"
-        if len(shape) == 2:
+        if leaf == "dwa":  # close to "hand on the newest result"
+            w = 0.1 * torch.randn(shape, generator=g) / shape[0]
+            w[-1] += 1.0
+        elif len(shape) == 2:
             std = 0.5 if name == "embed" else 1.0 / math.sqrt(shape[1])
             w = torch.randn(shape, generator=g) * std
-        elif leaf in ("norm", "norm1") or name == "final.norm":
+        elif leaf in ("norm", "norm1", "norm2") or name == "final.norm":
             w = 1.0 + 0.1 * torch.randn(shape, generator=g)
         else:
             w = 0.3 * torch.randn(shape, generator=g)

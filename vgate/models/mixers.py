@@ -10,6 +10,13 @@ spec, so another design can reuse a mixer with other values.
   are absorbed into the query and the output.
 * :class:`GeneralDelta` — generalized delta rule with per-channel decay over an fp32 state matrix
   per head, kept in a state slot per sequence.
+* :class:`WindowAttention` — grouped-query attention over a sliding window of a paged key/value cache,
+  optionally with one mean key / value per block of tokens that has left the window, a sink in the
+  softmax denominator, query / key norms over the head or the whole projection, values rotated by
+  their position.
+* :class:`LinearAttention` — decayed outer-product recurrence S <- diag(a) S + k v^T, o = S^T q over an
+  fp32 state per head in a state slot; the decay is a constant per head or a gated value per key channel.
+* :class:`ParallelMixers` — two mixers reading the same input, their outputs added with fixed scales.
 * :class:`DenseFF`, :class:`MoEFF` — gated feed-forward; sigmoid-routed mixture of clamped gated experts.
 """
 from __future__ import annotations
@@ -32,19 +39,25 @@ PACKED_MIN_K = 512
 class Proj:
     """y = x W^T for a [N, K] matrix, on whichever GEMM takes its shape and dtype."""
 
-    def __init__(self, w: torch.Tensor, device, f32: bool, silu_pair: bool = False, allow_packed: bool = True):
+    def __init__(self, w: torch.Tensor, device, f32: bool, silu_pair: bool = False, allow_packed: bool = True,
+                 bias: torch.Tensor | None = None, pair_act: int = seq.ACT_SILU_MUL):
         N, K = w.shape
         self.N, self.K, self.f32, self.silu_pair = N, K, f32, silu_pair
+        self.pair_act = pair_act
         dev = torch.device(device)
         n_ok = (N // 2) % 64 == 0 if silu_pair else N % 64 == 0
+        # the packed kernels' pair epilogue is SiLU; another pair activation runs on the row-major GEMM
         self.packed = (USE_PACKED and allow_packed and not f32 and dev.type == "cuda" and n_ok and K % 64 == 0
-                       and K >= PACKED_MIN_K)
+                       and K >= PACKED_MIN_K and (not silu_pair or pair_act == seq.ACT_SILU_MUL))
+        self.bias = None
         if self.packed:
-            self.lin = ops.Linear(w.to(dev, torch.bfloat16), kind="silu" if silu_pair else "plain")
+            self.lin = ops.Linear(w.to(dev, torch.bfloat16), kind="silu" if silu_pair else "plain",
+                                  bias=None if bias is None else bias.to(dev, torch.bfloat16).contiguous())
             self.w = None
         else:
             self.lin = None
             self.w = w.to(dev, torch.float32 if f32 else torch.bfloat16).contiguous()
+            self.bias = None if bias is None else bias.to(dev, torch.float32).contiguous()
         self.out_features = N // 2 if silu_pair else N
 
     def nbytes(self) -> int:
@@ -59,8 +72,8 @@ class Proj:
             out = torch.empty(M, self.out_features, dtype=dt, device=x.device)
         if self.silu_pair:
             I = self.N // 2
-            return seq.gemm(x, self.w[:I], out, w2=self.w[I:], act=seq.ACT_SILU_MUL)
-        return seq.gemm(x, self.w, out, act=act)
+            return seq.gemm(x, self.w[:I], out, w2=self.w[I:], act=self.pair_act)
+        return seq.gemm(x, self.w, out, act=act, bias=self.bias)
 
 
 def _f32(t: torch.Tensor, device) -> torch.Tensor:
@@ -95,6 +108,7 @@ class LatentAttention:
         H, D, R, V, KR = self.H, self.D, self.R, self.V, self.KR
         self.inv_freq = seq.rope_inv_freq(dims, float(rot.get("base", 10000.0)), dev)  # base^(-2i / dims)
         self.in_rows = [("dq", tensors["dq"]), ("dkv", tensors["dkv"]), ("g", tensors["g"])]
+        self.in_bias = {}
         self.dq_norm, self.dkv_norm = _f32(tensors["dq.norm"], dev), _f32(tensors["dkv.norm"], dev)
         self.uq = Proj(tensors["uq"], dev, f32)
         dt = torch.float32 if f32 else torch.bfloat16
@@ -126,6 +140,12 @@ class LatentAttention:
 
     def cache_dtype(self):
         return torch.float32 if self.f32 else torch.bfloat16
+
+    def allocate(self, num_blocks: int, block_size: int, num_slots: int, device) -> torch.Tensor:
+        return torch.zeros(self.cache_shape(num_blocks, block_size, num_slots), dtype=self.cache_dtype(), device=device)
+
+    def page_bytes(self, block_size: int) -> int:
+        return math.prod(self.cache_shape(1, block_size, 1)) * (4 if self.f32 else 2)
 
     def nbytes(self) -> int:
         return self.uq.nbytes() + self.o.nbytes() + 2 * self.uk_t.numel() * self.uk_t.element_size()
@@ -170,6 +190,9 @@ class GeneralDelta:
         self.unit_eps = self.UNIT_EPS if unit_eps is None else unit_eps
         dev = torch.device(device)
         self.in_rows = [(n, tensors[n]) for n in ("r", "k", "v", "g", "a")]
+        self.in_bias = {}
+        if tensors["w2"].shape[1] != tensors["w1"].shape[0]:
+            raise ValueError("general_delta: w1 / w2 disagree on the decay's width")
         self.w1 = Proj(tensors["w1"], dev, f32, allow_packed=False)  # tanh in its epilogue
         self.w2 = Proj(tensors["w2"], dev, f32)
         self.w0, self.ab, self.nw = _f32(tensors["w0"], dev), _f32(tensors["a.b"], dev), _f32(tensors["norm"], dev)
@@ -178,15 +201,21 @@ class GeneralDelta:
     @staticmethod
     def shapes(spec: dict, width: int) -> dict:
         n = spec["heads"] * spec["dim"]
-        decay_rank = int(spec.get("decay_rank", 16))  # checkpoints: the shape of w1 gives it
+        # None: the decay's low-rank width, which only the checkpoint's tensors give
         return {"r": (n, width), "k": (n, width), "v": (n, width), "g": (n, width), "a": (n, width), "a.b": (n,),
-                "w1": (decay_rank, width), "w2": (n, decay_rank), "w0": (n,), "norm": (n,), "o": (width, n)}
+                "w1": (None, width), "w2": (n, None), "w0": (n,), "norm": (n,), "o": (width, n)}
 
     def cache_shape(self, num_blocks: int, block_size: int, num_slots: int) -> tuple:
         return (num_slots, self.H, self.D, self.D)
 
     def cache_dtype(self):
         return torch.float32
+
+    def allocate(self, num_blocks: int, block_size: int, num_slots: int, device) -> torch.Tensor:
+        return torch.zeros(self.cache_shape(num_blocks, block_size, num_slots), dtype=torch.float32, device=device)
+
+    def page_bytes(self, block_size: int) -> int:
+        return 0
 
     def nbytes(self) -> int:
         return self.w1.nbytes() + self.w2.nbytes() + self.o.nbytes()
@@ -201,15 +230,226 @@ class GeneralDelta:
         return self.o(out)
 
 
-MIXERS = {c.kind: c for c in (LatentAttention, GeneralDelta)}
+class WindowAttention:
+    """Grouped-query attention over the last ``window`` positions of a paged key/value cache.
+
+    spec: heads, kv_heads, dim, vdim, scale, rot {base, dims, scaling}, window, and the options
+    ``pool`` (P > 0: every block of P tokens that lies wholly before the window is seen through the
+    mean of its cached keys and the mean of its cached values; tokens between such a block and the
+    window are not seen), ``qk_norm`` ("none" | "head": RMS norm per head with one [dim] weight |
+    "all": one RMS norm over the whole projection with a [heads * dim] weight), ``rotate_values``
+    (the cached value of position j is turned by j in pairs over all of vdim, the attention output
+    of position i is turned back by i), ``sink`` (one learned logit per head that only enters the
+    softmax denominator), ``bias`` (q / k / v biases), ``out_bias``.
+    """
+    kind = "window_attention"
+    cache = "paged"
+
+    def __init__(self, spec: dict, width: int, eps: float, tensors: dict, device, f32: bool):
+        m = spec
+        self.H, self.G, self.D, self.V = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
+        if self.G < 1 or self.H % self.G:
+            raise ValueError("window_attention: heads must be a multiple of kv_heads")
+        self.scale, self.window, self.pool = float(m["scale"]), int(m["window"]), int(m.get("pool") or 0)
+        if self.window < 1 or self.pool < 0:
+            raise ValueError("window_attention: window >= 1, pool >= 0")
+        self.qk_norm = m.get("qk_norm", "none")
+        if self.qk_norm not in ("none", "head", "all"):
+            raise ValueError(f"window_attention: qk_norm {self.qk_norm!r}")
+        rot = m.get("rot") or {}
+        dims = int(rot.get("dims", 0))
+        if dims > self.D or dims < 0:
+            raise ValueError("window_attention: rot.dims must be <= dim")
+        self.rot_dims = 2 * (dims // 2)
+        self.eps, self.f32 = eps, f32
+        dev = torch.device(device)
+        base = float(rot.get("base", 10000.0))
+        self.inv_freq = seq.rope_inv_freq(dims, base, dev, scaling=rot.get("scaling"))
+        self.v_freq = seq.rope_inv_freq(self.V, base, dev) if m.get("rotate_values") else None
+        self.in_rows = [(n, tensors[n]) for n in ("q", "k", "v")]
+        self.in_bias = {n: tensors[n + ".b"] for n in ("q", "k", "v")} if m.get("bias") else {}
+        self.qw = self.kw = None
+        if self.qk_norm != "none":
+            self.qw, self.kw = _f32(tensors["q.norm"], dev), _f32(tensors["k.norm"], dev)
+        self.sink = _f32(tensors["sink"], dev) if m.get("sink") else None
+        self.o = Proj(tensors["o"], dev, f32, bias=tensors["o.b"] if m.get("out_bias") else None)
+
+    @staticmethod
+    def shapes(spec: dict, width: int) -> dict:
+        H, G, D, V = spec["heads"], spec["kv_heads"], spec["dim"], spec["vdim"]
+        out = {"q": (H * D, width), "k": (G * D, width), "v": (G * V, width), "o": (width, H * V)}
+        if spec.get("bias"):
+            out.update({"q.b": (H * D,), "k.b": (G * D,), "v.b": (G * V,)})
+        if spec.get("qk_norm", "none") == "head":
+            out.update({"q.norm": (D,), "k.norm": (D,)})
+        elif spec.get("qk_norm") == "all":
+            out.update({"q.norm": (H * D,), "k.norm": (G * D,)})
+        if spec.get("sink"):
+            out["sink"] = (H,)
+        if spec.get("out_bias"):
+            out["o.b"] = (width,)
+        return out
+
+    def pooled_per_page(self, block_size: int) -> int:
+        """Pooled rows a cache page carries: block b's means live in the page of its last position
+        b P + P - 1, in row (that position mod page) / P."""
+        return (block_size + self.pool - 1) // self.pool if self.pool else 0
+
+    def allocate(self, num_blocks: int, block_size: int, num_slots: int, device) -> tuple:
+        dt = torch.float32 if self.f32 else torch.bfloat16
+        npool = self.pooled_per_page(block_size)
+        z = lambda rows, d: torch.zeros(num_blocks, self.G, rows, d, dtype=dt, device=device)  # noqa: E731
+        return (z(block_size, self.D), z(block_size, self.V),
+                z(npool, self.D) if npool else None, z(npool, self.V) if npool else None)
+
+    def page_bytes(self, block_size: int) -> int:
+        return (block_size + self.pooled_per_page(block_size)) * self.G * (self.D + self.V) * (4 if self.f32 else 2)
+
+    def nbytes(self) -> int:
+        return self.o.nbytes()
+
+    def forward(self, h, P, cols, sv, cache) -> torch.Tensor:
+        T = h.shape[0]
+        kc, vc, kp, vp = cache
+        q = torch.empty(T, self.H * self.D, dtype=h.dtype, device=h.device)
+        seq.window_write(cols(P, "q"), cols(P, "k"), cols(P, "v"), self.qw, self.kw, self.eps, self.qk_norm == "all",
+                         sv.positions, sv.slots, self.inv_freq, self.rot_dims, self.v_freq, kc, vc, q, self.H, self.G)
+        if self.pool:
+            seq.window_pool(kc, vc, kp, vp, sv.positions, sv.block_tables, sv.query_start, self.pool,
+                            num_seqs=sv.num_seqs or None)
+        o = torch.empty(T, self.H * self.V, dtype=h.dtype, device=h.device)
+        seq.window_attn(q, kc, vc, kp, vp, sv.block_tables, sv.context_lens, sv.query_start, o, self.scale, self.H,
+                        self.window, self.pool, self.sink, self.v_freq, num_seqs=sv.num_seqs or None)
+        return self.o(o, out_f32=True)
+
+
+class LinearAttention:
+    """Decayed outer-product recurrence per head over an fp32 state [dim, vdim] in a state slot:
+    S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T (q_scale q_t).
+
+    spec: heads, dim, vdim, ``decay`` ({"kind": "head", "values": [one constant per head]} or
+    {"kind": "channel", "tau": tau}: a = sigmoid(z)^(1 / tau) per key channel with z = W_a2 (W_a1 h) +
+    b, a low-rank gate whose width the checkpoint's tensors give), ``q_scale``, ``in_act`` ("none" |
+    "silu" on q, k and v), ``out_norm`` ("head": RMS norm per head with one [vdim] weight | "all":
+    over the concatenated heads with a [heads * vdim] weight), ``gate_act`` ("silu" | "sigmoid" of
+    W_g h, multiplied onto the normed output before the output projection).
+    """
+    kind = "linear_attention"
+    cache = "state"
+
+    def __init__(self, spec: dict, width: int, eps: float, tensors: dict, device, f32: bool):
+        self.H, self.D, self.V = int(spec["heads"]), int(spec["dim"]), int(spec["vdim"])
+        if self.D > seq.LINEAR_ATTN_MAX_DIM:
+            raise ValueError(f"linear_attention: the recurrence keeps a state column in registers: dim <= {seq.LINEAR_ATTN_MAX_DIM}")
+        self.eps, self.f32 = eps, f32
+        dev = torch.device(device)
+        dec = spec["decay"]
+        self.channel = dec["kind"] == "channel"
+        if dec["kind"] not in ("channel", "head"):
+            raise ValueError(f"linear_attention: decay kind {dec['kind']!r}")
+        for key, allowed in (("in_act", ("none", "silu")), ("out_norm", ("head", "all")), ("gate_act", ("silu", "sigmoid"))):
+            if spec[key] not in allowed:
+                raise ValueError(f"linear_attention: {key} {spec[key]!r}")
+        self.q_scale = float(spec.get("q_scale", 1.0))
+        self.in_silu, self.norm_all, self.gate_silu = spec["in_act"] == "silu", spec["out_norm"] == "all", spec["gate_act"] == "silu"
+        self.in_rows = [(n, tensors[n]) for n in ("q", "k", "v", "g")]
+        self.in_bias = {}
+        self.tau, self.a2, self.head_decay = 1.0, None, None
+        if self.channel:
+            self.tau = float(dec["tau"])
+            if tensors["a2"].shape[1] != tensors["a1"].shape[0]:
+                raise ValueError("linear_attention: a1 / a2 disagree on the gate's width")
+            self.in_rows.append(("a1", tensors["a1"]))
+            self.a2 = Proj(tensors["a2"], dev, f32, allow_packed=False, bias=tensors["a2.b"])  # fp32 gate logits
+        else:
+            self.head_decay = torch.tensor([float(d) for d in dec["values"]], dtype=torch.float32, device=dev)
+        self.nw = _f32(tensors["norm"], dev)
+        self.o = Proj(tensors["o"], dev, f32)
+
+    @staticmethod
+    def shapes(spec: dict, width: int) -> dict:
+        H, D, V = spec["heads"], spec["dim"], spec["vdim"]
+        out = {"q": (H * D, width), "k": (H * D, width), "v": (H * V, width), "g": (H * V, width), "o": (width, H * V),
+               "norm": (H * V,) if spec["out_norm"] == "all" else (V,)}
+        if spec["decay"]["kind"] == "channel":  # None: the gate's width, which only the tensors give
+            out.update({"a1": (None, width), "a2": (H * D, None), "a2.b": (H * D,)})
+        return out
+
+    def allocate(self, num_blocks: int, block_size: int, num_slots: int, device) -> torch.Tensor:
+        return torch.zeros(num_slots, self.H, self.D, self.V, dtype=torch.float32, device=device)
+
+    def page_bytes(self, block_size: int) -> int:
+        return 0
+
+    def nbytes(self) -> int:
+        return self.o.nbytes() + (self.a2.nbytes() if self.a2 else 0)
+
+    def forward(self, h, P, cols, sv, cache) -> torch.Tensor:
+        T = h.shape[0]
+        z = self.a2(cols(P, "a1"), out_f32=True) if self.channel else None
+        out = torch.empty(T, self.H * self.V, dtype=h.dtype, device=h.device)
+        seq.linear_attn(cols(P, "q"), cols(P, "k"), cols(P, "v"), cols(P, "g"), z, self.head_decay, self.tau, self.q_scale,
+                        self.in_silu, self.nw, self.norm_all, self.gate_silu, cache, sv.state_slots, sv.context_lens,
+                        sv.query_start, out, self.eps, num_seqs=sv.num_seqs or None)
+        return self.o(out, out_f32=True)
+
+
+class ParallelMixers:
+    """Two mixers side by side on the same input: y = left_scale * left(h) + right_scale * right(h).
+    spec: ``left`` / ``right`` = (key of MIXERS, that mixer's spec); tensors under ``left.`` / ``right.``.
+    ``forward`` returns the two outputs with their scales; the layer's residual kernel adds them."""
+    kind = "parallel"
+    cache = "both"
+
+    def __init__(self, spec: dict, width: int, eps: float, tensors: dict, device, f32: bool):
+        self.parts, self.scales = [], (float(spec["left_scale"]), float(spec["right_scale"]))
+        self.in_rows, self.in_bias = [], {}
+        for side in ("left", "right"):
+            kind, sub_spec = spec[side]
+            t = {k[len(side) + 1:]: v for k, v in tensors.items() if k.startswith(side + ".")}
+            mx = MIXERS[kind](sub_spec, width, eps, t, device, f32)
+            self.in_rows += [(f"{side}.{n}", w) for n, w in mx.in_rows]
+            self.in_bias.update({f"{side}.{n}": b for n, b in mx.in_bias.items()})
+            del mx.in_rows
+            self.parts.append((side, mx))
+
+    @staticmethod
+    def shapes(spec: dict, width: int) -> dict:
+        out = {}
+        for side in ("left", "right"):
+            kind, sub_spec = spec[side]
+            out.update({f"{side}.{k}": v for k, v in MIXERS[kind].shapes(sub_spec, width).items()})
+        return out
+
+    def allocate(self, num_blocks: int, block_size: int, num_slots: int, device) -> tuple:
+        return tuple(mx.allocate(num_blocks, block_size, num_slots, device) for _, mx in self.parts)
+
+    def page_bytes(self, block_size: int) -> int:
+        return sum(mx.page_bytes(block_size) for _, mx in self.parts)
+
+    def nbytes(self) -> int:
+        return sum(mx.nbytes() for _, mx in self.parts)
+
+    def forward(self, h, P, cols, sv, cache) -> tuple:
+        ys = [mx.forward(h, P, (lambda P_, n, s=side: cols(P_, f"{s}.{n}")), sv, c)
+              for (side, mx), c in zip(self.parts, cache)]
+        return ys[0], self.scales[0], ys[1], self.scales[1]
+
+
+MIXERS = {c.kind: c for c in (LatentAttention, GeneralDelta, WindowAttention, LinearAttention, ParallelMixers)}
 
 
 # ------------------------------------------------------------------------------------ feed-forwards
 class DenseFF:
-    """down(silu(gate h) * (up h))."""
+    """down(act(gate h) * (up h)); spec ``act``: "silu" (default) or "gelu_tanh"."""
+    ACTS = {"silu": seq.ACT_SILU_MUL, "gelu_tanh": seq.ACT_GELU_TANH_MUL}
 
     def __init__(self, spec: dict, width: int, tensors: dict, device, f32: bool):
-        self.gate_up = Proj(torch.cat([tensors["gate"], tensors["up"]]), device, f32, silu_pair=True)
+        act = spec.get("act", "silu")
+        if act not in self.ACTS:
+            raise ValueError(f"dense feed-forward: act {act!r}")
+        self.gate_up = Proj(torch.cat([tensors["gate"], tensors["up"]]), device, f32, silu_pair=True,
+                            pair_act=self.ACTS[act])
         self.down = Proj(tensors["down"], device, f32)
 
     @staticmethod
@@ -219,8 +459,8 @@ class DenseFF:
     def nbytes(self) -> int:
         return self.gate_up.nbytes() + self.down.nbytes()
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
-        return self.down(self.gate_up(h))
+    def forward(self, h: torch.Tensor, out_f32: bool = False) -> torch.Tensor:
+        return self.down(self.gate_up(h), out_f32=out_f32)
 
 
 class MoEFF:
@@ -274,18 +514,3 @@ class MoEFF:
 
 
 FEED_FORWARDS = {"dense": DenseFF, "moe": MoEFF}
-
-
-def layer_shapes(spec, width: int) -> dict:
-    """name -> shape of every tensor of a layer that owns its weights (suffixes after 'l<i>.')."""
-    out = {"norm1": ()}
-    out.update({"mix." + k: v for k, v in MIXERS[spec.kind].shapes(spec.mixer, width).items()})
-    out.update({"rg1": (width, width), "rg1.b": (width,)})
-    if spec.mlp:
-        out.update({"mlp." + k: v for k, v in FEED_FORWARDS[spec.mlp["kind"]].shapes(spec.mlp, width).items()})
-        out.update({"rg2": (width, width), "rg2.b": (width,)})
-    return out
-
-
-def layer_params(spec, width: int) -> int:
-    return sum(math.prod(s) for s in layer_shapes(spec, width).values())

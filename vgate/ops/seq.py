@@ -8,6 +8,7 @@ at the same places.
 """
 from __future__ import annotations
 
+import math
 import os
 
 import torch
@@ -41,7 +42,8 @@ def _C():
     return _Traced(mod) if _TRACE else mod
 
 
-ACT_NONE, ACT_SILU_MUL, ACT_CLAMPED_GLU, ACT_TANH = 0, 1, 2, 3
+ACT_NONE, ACT_SILU_MUL, ACT_CLAMPED_GLU, ACT_TANH, ACT_GELU_TANH_MUL = 0, 1, 2, 3, 4
+LINEAR_ATTN_MAX_DIM = 256   # key channels per head the recurrence kernel keeps in registers (csrc/kernels/linear_attn.hip)
 
 
 def _act(g: torch.Tensor, u: torch.Tensor | None, act: int, limit: float, alpha: float) -> torch.Tensor:
@@ -53,6 +55,8 @@ def _act(g: torch.Tensor, u: torch.Tensor | None, act: int, limit: float, alpha:
         return g * torch.sigmoid(alpha * g) * (u + 1.0)
     if act == ACT_TANH:
         return torch.tanh(g)
+    if act == ACT_GELU_TANH_MUL:
+        return 0.5 * g * (1.0 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g * g * g))) * u
     return g
 
 
@@ -133,10 +137,24 @@ def gated_residual(x, y1, g1=None, b1=None, y2=None, g2=None, b2=None) -> None:
     x += v
 
 
-def rope_inv_freq(dims: int, base: float, device) -> torch.Tensor:
-    """f_i = base^(-2i / dims), i < dims / 2, in fp32."""
-    i = torch.arange(dims // 2, dtype=torch.float32)
-    return (base ** (-2.0 * i / dims)).to(torch.float32).to(device)
+def rope_inv_freq(dims: int, base: float, device, scaling: dict | None = None) -> torch.Tensor:
+    """f_i = base^(-2i / dims), i < dims / 2, rounded to fp32 once. ``scaling`` {factor, low, high,
+    original} stretches long wavelengths (the Llama-3.1 rule): with l = 2 pi / f, f is kept where
+    l < original / high, divided by factor where l > original / low, and blended linearly in
+    original / l between the two."""
+    out = []
+    for i in range(dims // 2):
+        f = float(base) ** (-2.0 * i / dims)
+        if scaling:
+            factor, low, high, orig = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+            wl = 2.0 * math.pi / f
+            if wl > orig / low:
+                f = f / factor
+            elif wl >= orig / high:
+                s = (orig / wl - low) / (high - low)
+                f = (1.0 - s) * f / factor + s * f
+        out.append(f)
+    return torch.tensor(out, dtype=torch.float32).to(device)
 
 
 def _rope_pairs(x: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor, dims: int) -> torch.Tensor:
@@ -284,3 +302,193 @@ def moe_combine(y, pos, wts, out) -> None:
     T, top = wts.shape
     rows = y.float()[pos.view(T, top).long()]
     out.copy_((rows * wts[:, :, None]).sum(1))
+
+
+# ------------------------------------------------------------------ post-norm residual, depth average
+def cast_rows(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = x rounded to out's dtype (the copy of the fp32 stream a bf16 GEMM reads)."""
+    if x.is_cuda:
+        _C().cast_rows(x, out)
+        return out
+    out.copy_(x[: out.shape[0]])
+    return out
+
+
+def post_norm_add(x, y1, w, eps: float, out, s1: float = 1.0, y2=None, s2: float = 1.0, act_out=None, hist=None,
+                  planes: int = 0, coef=None, mix=None) -> None:
+    """out = x + u / sqrt(mean(u^2) + eps) * w with u = s1 y1 [+ s2 y2], all in fp32 (out may be x).
+    With ``hist`` [n, T, W] (whose plane ``planes - 1`` is ``out``): mix = sum_{j < planes} coef[j] hist[j],
+    the depth average. ``act_out``: a copy of mix (or of out without hist) in the activation dtype."""
+    if x.is_cuda:
+        _C().post_norm_add(x, y1, w, eps, out, s1, y2, s2, act_out, hist, planes, coef, mix)
+        return
+    T = out.shape[0]
+    u = y1[:T].float() * s1
+    if y2 is not None:
+        u = u + y2[:T].float() * s2
+    r = x[:T] + u * (1.0 / torch.sqrt(u.pow(2).mean(-1, keepdim=True) + eps)) * w
+    out.copy_(r)
+    last = out
+    if hist is not None:
+        acc = torch.zeros_like(r)
+        for j in range(planes):
+            acc = acc + coef[j] * hist[j][:T]
+        mix.copy_(acc)
+        last = mix
+    if act_out is not None:
+        act_out.copy_(last)
+
+
+# ---------------------------------------------------------------------------------- window attention
+def _rope_pairs_heads(x: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor, dims: int, sign: float = 1.0):
+    """x [T, heads, d]: the leading ``dims`` entries of every head turned in interleaved pairs by sign * pos * f_i."""
+    return _rope_pairs(x, pos.float() * sign, inv_freq, dims)
+
+
+def window_write(q, k, v, qw, kw, eps: float, norm_all: bool, positions, slots, inv_freq, rot_dims: int, v_freq,
+                 kc, vc, q_out, H: int, G: int) -> None:
+    """Prepare one step's queries, keys and values of a window-attention layer.
+    q [T, H * D], k [T, G * D], v [T, G * V] (biases already added). Query / key RMS norm (``qw`` / ``kw``
+    None: none; ``norm_all``: over the whole projection with a [heads * D] weight, else per head with a
+    [D] weight), rotation of the first ``rot_dims`` entries of every head, values turned over all of V
+    by ``v_freq`` if given. q goes to ``q_out``; keys and values to the paged caches
+    kc [pages, G, page, D] / vc [pages, G, page, V] at the tokens' slots (slot < 0: padding row)."""
+    if q.is_cuda:
+        _C().window_write(q, k, v, qw, kw, eps, norm_all, positions, slots, inv_freq, rot_dims, v_freq, kc, vc, q_out, H, G)
+        return
+    T = q.shape[0]
+    D, V, page = kc.shape[3], vc.shape[3], kc.shape[2]
+    qf, kf, vf = q.float(), k.float(), v.float()
+
+    def norm(x, w, heads):
+        if w is None:
+            return x.view(T, heads, D)
+        if norm_all:
+            return (x * (1.0 / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps)) * w).view(T, heads, D)
+        x = x.view(T, heads, D)
+        return x * (1.0 / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps)) * w
+
+    qn = _rope_pairs_heads(norm(qf, qw, H), positions[:T], inv_freq, rot_dims)
+    kn = _rope_pairs_heads(norm(kf, kw, G), positions[:T], inv_freq, rot_dims)
+    vn = vf.view(T, G, V)
+    if v_freq is not None:
+        vn = _rope_pairs_heads(vn, positions[:T], v_freq, 2 * v_freq.numel())
+    q_out.copy_(qn.reshape(T, H * D))
+    ok = slots[:T] >= 0
+    sl = slots[:T][ok].long()
+    kc[sl // page, :, sl % page] = kn[ok].to(kc.dtype)
+    vc[sl // page, :, sl % page] = vn[ok].to(vc.dtype)
+
+
+def _seq_rows(block_table: torch.Tensor, j: torch.Tensor, page: int):
+    return block_table.long()[j // page], j % page
+
+
+def window_pool(kc, vc, kp, vp, positions, block_tables, query_start, pool: int, num_seqs: int | None = None) -> None:
+    """For every token of the step whose position completes a block of ``pool`` tokens: the mean of the
+    block's cached keys (values) goes to kp (vp) [pages, G, ceil(page / pool), D], into the page of the
+    block's last position e, row (e mod page) / pool."""
+    if kc.is_cuda:
+        _C().window_pool(kc, vc, kp, vp, positions, block_tables, query_start, pool)
+        return
+    page = kc.shape[2]
+    S = block_tables.shape[0] if num_seqs is None else num_seqs
+    for s in range(S):
+        for t in range(int(query_start[s]), int(query_start[s + 1])):
+            e = int(positions[t])
+            if (e + 1) % pool:
+                continue
+            pg, r = _seq_rows(block_tables[s], torch.arange(e + 1 - pool, e + 1), page)
+            dst = int(block_tables[s][e // page])
+            kp[dst, :, (e % page) // pool] = kc[pg, :, r].float().mean(0).to(kp.dtype)
+            vp[dst, :, (e % page) // pool] = vc[pg, :, r].float().mean(0).to(vp.dtype)
+
+
+def window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out, scale: float, H: int, window: int,
+                pool: int, sink, v_freq, num_seqs: int | None = None) -> None:
+    """out[t, h] = sum_j p_j value_j over the keys position i of token t sees: the tokens j with
+    0 <= i - j < window and, with ``pool`` = P > 0, the pooled row of every block b with
+    b P + P - 1 <= i - window; p = softmax(scale q . key) over both kinds together, with exp(sink[h]) added
+    to the denominator if ``sink`` is given. With ``v_freq`` the result is turned back by -i over all of V.
+    Query head h reads key/value head h / (H / G)."""
+    if q.is_cuda:
+        _C().window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out, scale, H, window, pool, sink, v_freq)
+        return
+    G, page, D, V = kc.shape[1], kc.shape[2], kc.shape[3], vc.shape[3]
+    rep = H // G
+    S = block_tables.shape[0] if num_seqs is None else num_seqs
+    for s in range(S):
+        t0, t1 = int(query_start[s]), int(query_start[s + 1])
+        if t1 <= t0:
+            continue
+        pos0 = int(context_lens[s]) - (t1 - t0)
+        bt = block_tables[s]
+        for t in range(t0, t1):
+            i = pos0 + t - t0
+            lo = max(0, i - window + 1)
+            pg, r = _seq_rows(bt, torch.arange(lo, i + 1), page)
+            K, Vv = kc[pg, :, r].float(), vc[pg, :, r].float()           # [n, G, D], [n, G, V]
+            nb = max(0, i - window + 1) // pool if pool else 0
+            if nb:
+                e = torch.arange(nb) * pool + pool - 1
+                pg, r = _seq_rows(bt, e, page)
+                K = torch.cat([kp[pg, :, r // pool].float(), K])
+                Vv = torch.cat([vp[pg, :, r // pool].float(), Vv])
+            qh = q[t].float().view(G, rep, D)
+            sc = torch.einsum("grd,ngd->grn", qh, K) * scale               # [G, rep, n]
+            if sink is not None:
+                sc = torch.cat([sc, sink.view(G, rep, 1)], -1)
+            p = torch.softmax(sc, -1)[..., : K.shape[0]]
+            o = torch.einsum("grn,ngv->grv", p, Vv).reshape(1, H, V)
+            if v_freq is not None:
+                o = _rope_pairs(o, torch.tensor([-float(i)]), v_freq, 2 * v_freq.numel())
+            out[t] = o.reshape(H * V).to(out.dtype)
+
+
+# ---------------------------------------------------------------------------------- linear attention
+def linear_attn(q, k, v, g, z, head_decay, tau: float, q_scale: float, in_silu: bool, nw, norm_all: bool,
+                gate_silu: bool, state, state_slots, context_lens, query_start, out, eps: float,
+                num_seqs: int | None = None) -> None:
+    """Decayed outer-product recurrence over state slots, state [slots, H, D, V] fp32:
+        S <- diag(a_t) S + k_t v_t^T,  o_t = S^T (q_scale q_t)
+    a_t = sigmoid(z_t)^(1 / tau) per key channel (``z`` fp32 [T, H * D]) or the constant head_decay[h];
+    ``in_silu``: silu on q, k, v. Then RMS norm of o (per head with a [V] weight, or with ``norm_all`` over
+    the concatenated heads with a [H * V] weight), times silu(g) or sigmoid(g). A portion that starts at
+    position 0 starts from a zero state."""
+    if q.is_cuda:
+        H, D, V = state.shape[1], state.shape[2], state.shape[3]
+        scratch = torch.empty(q.shape[0] * H * (4 * D + 2 * V), dtype=torch.float32, device=q.device)
+        _C().linear_attn(q, k, v, g, z, head_decay, tau, q_scale, in_silu, nw, norm_all, gate_silu, state, state_slots,
+                         context_lens, query_start, out, eps, scratch)
+        return
+    H, D, V = state.shape[1], state.shape[2], state.shape[3]
+    S = state_slots.numel() if num_seqs is None else num_seqs
+    act = torch.nn.functional.silu if in_silu else (lambda x: x)
+    for s in range(S):
+        t0, t1 = int(query_start[s]), int(query_start[s + 1])
+        slot = int(state_slots[s])
+        if t1 <= t0 or slot < 0:
+            continue
+        n = t1 - t0
+        pos0 = int(context_lens[s]) - n
+        St = state[slot].clone() if pos0 > 0 else torch.zeros(H, D, V)
+        qq = act(q[t0:t1].float()).view(n, H, D) * q_scale
+        kk = act(k[t0:t1].float()).view(n, H, D)
+        vv = act(v[t0:t1].float()).view(n, H, V)
+        if z is not None:
+            a = torch.exp(torch.nn.functional.logsigmoid(z[t0:t1].float()) / tau).view(n, H, D)
+        else:
+            a = head_decay.view(1, H, 1).expand(n, H, D)
+        o = torch.empty(n, H, V)
+        for i in range(n):
+            St = a[i][:, :, None] * St + kk[i][:, :, None] * vv[i][:, None, :]
+            o[i] = torch.einsum("hdv,hd->hv", St, qq[i])
+        state[slot] = St
+        if norm_all:
+            of = o.reshape(n, H * V)
+            of = of * (1.0 / torch.sqrt(of.pow(2).mean(-1, keepdim=True) + eps)) * nw
+        else:
+            of = (o * (1.0 / torch.sqrt(o.pow(2).mean(-1, keepdim=True) + eps)) * nw).reshape(n, H * V)
+        gg = g[t0:t1].float()
+        of = of * (torch.nn.functional.silu(gg) if gate_silu else torch.sigmoid(gg))
+        out[t0:t1] = of.to(out.dtype)
