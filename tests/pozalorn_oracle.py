@@ -58,45 +58,63 @@ def turn_pairs(x: torch.Tensor, pos: float, freqs: torch.Tensor, n_dims: int) ->
 
 
 # -------------------------------------------------------------------------------------------- mixers
+def recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tensor, S: torch.Tensor | None = None):
+    """One head: S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t. q, k, a [T, D]; v [T, V]. Returns (o, S)."""
+    T, D = q.shape
+    S = torch.zeros(D, v.shape[1], dtype=q.dtype) if S is None else S.clone()
+    o = []
+    for t in range(T):
+        S = a[t][:, None] * S + k[t][:, None] * v[t][None, :]
+        o.append(S.t() @ q[t])
+    return torch.stack(o), S
+
+
+def attend(q: torch.Tensor, keys: list, vals: list, t: int, size: int, pool: int, scale: float, sink) -> torch.Tensor:
+    """Position t's attention output [H, V]: q [H, D]; keys[j] [G, D] and vals[j] [G, V] of positions 0 .. t."""
+    H, G = q.shape[0], keys[0].shape[0]
+    ks, vs = [], []
+    if pool:
+        b = 0
+        while b * pool + pool - 1 <= t - size:
+            ks.append(torch.stack(keys[b * pool: b * pool + pool]).mean(0))
+            vs.append(torch.stack(vals[b * pool: b * pool + pool]).mean(0))
+            b += 1
+    lo = max(0, t - size + 1)
+    K, V = torch.stack(ks + keys[lo: t + 1]), torch.stack(vs + vals[lo: t + 1])   # [n, G, D], [n, G, Dv]
+    o = torch.zeros(H, V.shape[-1], dtype=q.dtype)
+    for hd in range(H):
+        g = hd // (H // G)
+        sc = (K[:, g] @ q[hd]) * scale
+        mx = sc.max() if sink is None else torch.maximum(sc.max(), sink[hd])
+        e = torch.exp(sc - mx)
+        den = e.sum() + (torch.exp(sink[hd] - mx) if sink is not None else 0.0)
+        o[hd] = (e / den) @ V[:, g]
+    return o
+
+
 def gated_linear_attention(h: torch.Tensor, w: dict, m: dict, eps: float) -> torch.Tensor:
     """S_t = diag(alpha_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per head; alpha = sigmoid(z)^(1 / tau)."""
     H, D, Dv, tau = m["heads"], m["dim"], m["vdim"], float(m["tau"])
     T = h.shape[0]
-    out = []
-    S = torch.zeros(H, D, Dv, dtype=h.dtype)
-    for t in range(T):
-        x = h[t]
-        q = (w["q"] @ x).view(H, D) * D ** -0.5
-        k = (w["k"] @ x).view(H, D)
-        v = (w["v"] @ x).view(H, Dv)
-        z = (w["a2"] @ (w["a1"] @ x) + w["a2.b"]).view(H, D)
-        alpha = torch.sigmoid(z) ** (1.0 / tau)
-        o = torch.zeros(H, Dv, dtype=h.dtype)
-        for hd in range(H):
-            S[hd] = alpha[hd][:, None] * S[hd] + k[hd][:, None] * v[hd][None, :]
-            o[hd] = S[hd].t() @ q[hd]
-        o = rms_unit(o, eps) * w["norm"]            # per head, one weight vector for all heads
-        g = silu(w["g"] @ x)
-        out.append(w["o"] @ (o.reshape(-1) * g))
-    return torch.stack(out)
+    q = (h @ w["q"].t()).view(T, H, D) * D ** -0.5
+    k = (h @ w["k"].t()).view(T, H, D)
+    v = (h @ w["v"].t()).view(T, H, Dv)
+    z = ((h @ w["a1"].t()) @ w["a2"].t() + w["a2.b"]).view(T, H, D)
+    alpha = torch.sigmoid(z) ** (1.0 / tau)
+    o = torch.stack([recurrence(q[:, i], k[:, i], v[:, i], alpha[:, i])[0] for i in range(H)], 1)   # [T, H, Dv]
+    o = rms_unit(o, eps) * w["norm"]                # per head, one weight vector for all heads
+    return (o.reshape(T, -1) * silu(h @ w["g"].t())) @ w["o"].t()
 
 
 def lightning_attention(h: torch.Tensor, w: dict, m: dict, eps: float) -> torch.Tensor:
     """S_t = decay_h S_(t-1) + k_t v_t^T with silu on q, k, v; the heads are normed together."""
     H, D, Dv = m["heads"], m["dim"], m["vdim"]
-    decay = [float(d) for d in m["decay"]]
-    S = torch.zeros(H, D, Dv, dtype=h.dtype)
-    out = []
-    for t in range(h.shape[0]):
-        x = h[t]
-        q, k, v = silu(w["q"] @ x).view(H, D), silu(w["k"] @ x).view(H, D), silu(w["v"] @ x).view(H, Dv)
-        o = torch.zeros(H, Dv, dtype=h.dtype)
-        for hd in range(H):
-            S[hd] = decay[hd] * S[hd] + k[hd][:, None] * v[hd][None, :]
-            o[hd] = S[hd].t() @ q[hd]
-        o = rms_unit(o.reshape(-1), eps) * w["norm"]
-        out.append(w["o"] @ (o * torch.sigmoid(w["g"] @ x)))
-    return torch.stack(out)
+    T = h.shape[0]
+    q, k, v = silu(h @ w["q"].t()).view(T, H, D), silu(h @ w["k"].t()).view(T, H, D), silu(h @ w["v"].t()).view(T, H, Dv)
+    o = torch.stack([recurrence(q[:, i], k[:, i], v[:, i], torch.full((T, D), float(m["decay"][i]), dtype=h.dtype))[0]
+                     for i in range(H)], 1)
+    o = rms_unit(o.reshape(T, -1), eps) * w["norm"]
+    return (o * torch.sigmoid(h @ w["g"].t())) @ w["o"].t()
 
 
 def window_attention(h: torch.Tensor, w: dict, m: dict, eps: float, norm_over: str, turn_values: bool,
@@ -130,27 +148,9 @@ def window_attention(h: torch.Tensor, w: dict, m: dict, eps: float, norm_over: s
             v = torch.stack([turn_pairs(v[i], t, fv, Dv) for i in range(G)])
         keys.append(k)
         vals.append(v)
-        lo = max(0, t - size + 1)
-        ks, vs = [], []
-        if pool:
-            b = 0
-            while b * pool + pool - 1 <= t - size:
-                ks.append(torch.stack(keys[b * pool: b * pool + pool]).mean(0))
-                vs.append(torch.stack(vals[b * pool: b * pool + pool]).mean(0))
-                b += 1
-        ks += keys[lo: t + 1]
-        vs += vals[lo: t + 1]
-        K, V = torch.stack(ks), torch.stack(vs)            # [n, G, D], [n, G, Dv]
-        o = torch.zeros(H, Dv, dtype=h.dtype)
-        for hd in range(H):
-            g = hd // (H // G)
-            sc = (K[:, g] @ q[hd]) * float(m["scale"])
-            mx = sc.max() if sink is None else torch.maximum(sc.max(), sink[hd])
-            e = torch.exp(sc - mx)
-            den = e.sum() + (torch.exp(sink[hd] - mx) if sink is not None else 0.0)
-            o[hd] = (e / den) @ V[:, g]
-            if turn_values:
-                o[hd] = turn_pairs(o[hd], -t, fv, Dv)
+        o = attend(q, keys, vals, t, size, pool, float(m["scale"]), sink)
+        if turn_values:
+            o = torch.stack([turn_pairs(o[i], -t, fv, Dv) for i in range(H)])
         y = w["o"] @ o.reshape(-1)
         out.append(y + w["o.b"] if out_bias else y)
     return torch.stack(out)

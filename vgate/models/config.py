@@ -256,6 +256,27 @@ def _zadirax_preset(name: str, width: int, vocab: int, pairs: int, heads: int, d
     return HybridArch(name=name, family="zadirax", hidden_size=width, vocab_size=vocab, layers=tuple(layers))
 
 
+def _pozalorn_preset(name: str, width: int, vocab: int, groups: int, heads: int, kv_heads: int, dim: int, ff: int,
+                     window: int, pool: int, lin_heads: int | None = None) -> HybridArch:
+    """Random-init Pozalorn models (benchmarks, tests): ``groups`` x [gla, attention with pooled blocks,
+    sink attention beside lightning attention], each with a dense feed-forward."""
+    lh = lin_heads or heads
+    rot = {"base": 500000.0, "dims": dim, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    mlp = {"kind": "dense", "ff": ff}
+    gla = {"type": "gla", "mixer": {"heads": lh, "dim": dim, "vdim": dim, "tau": 16.0}, "mlp": mlp}
+    att = {"type": "attention", "mlp": mlp,
+           "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "rot": rot,
+                     "mask": {"size": window, "pool": pool}}}
+    par = {"type": "parallel", "mlp": mlp,
+           "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "rot": rot,
+                              "mask": {"size": window}},
+                     "right": {"heads": lh, "dim": dim, "vdim": dim,
+                               "decay": [math.exp(-(2.0 ** (-8.0 * (i + 1) / lh))) for i in range(lh)]},
+                     "left_scale": 1.0, "right_scale": 1.0}}
+    cfg = {"width": width, "vocab": vocab, "norm": {"eps": 1e-6}, "layers": [gla, att, par] * groups}
+    return _pozalorn_from_config(cfg, name)
+
+
 HYBRID_PRESETS = {
     # tests / CPU smoke: odd sizes on purpose (nothing a multiple of the MFMA tile)
     "zadirax-tiny": lambda: _zadirax_preset("zadirax-tiny", 96, 300, 2, 3, 24, 136, 5, 2, 40, 56, 40, 8, share=True),
@@ -263,6 +284,11 @@ HYBRID_PRESETS = {
     # equal width (benchmarks/design_compare.py)
     "zadirax-bench-1024": lambda: _zadirax_preset("zadirax-bench-1024", 1024, 32000, 2, 8, 128, 4096, 8, 2, 2048, 256, 512, 64),
     "zadirax-bench-1536": lambda: _zadirax_preset("zadirax-bench-1536", 1536, 32000, 2, 12, 128, 8960, 16, 4, 2240, 512, 768, 64),
+    # tests / CPU smoke: odd sizes on purpose
+    "pozalorn-tiny": lambda: _pozalorn_preset("pozalorn-tiny", 88, 300, 1, 4, 2, 24, 136, 21, 5, lin_heads=3),
+    # slices at the layer sizes of real models beside a transformer of equal width (benchmarks/design_compare.py)
+    "pozalorn-bench-1024": lambda: _pozalorn_preset("pozalorn-bench-1024", 1024, 32000, 1, 8, 2, 128, 4096, 1024, 64),
+    "pozalorn-bench-1536": lambda: _pozalorn_preset("pozalorn-bench-1536", 1536, 32000, 1, 12, 2, 128, 8960, 1024, 64),
     # layer sizes of a ~1.5B model (the width, head size, feed-forward and vocabulary of qwen2.5-1.5b)
     "zadirax-1.5b": lambda: _zadirax_preset("zadirax-1.5b", 1536, 151936, 14, 12, 128, 8960, 32, 4, 2240, 512, 768, 64),
 }
