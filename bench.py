@@ -356,8 +356,10 @@ def main():
                     default=float(os.environ.get("VGATE_SWITCH_INTERVAL_US", "0")),
                     help="sys.setswitchinterval for the server process (0 = Python default 5 ms)")
     ap.add_argument("--design-compare", action="store_true",
-                    help="instead of the serving benchmark: prefill / decode tokens/s of the Zadirax design beside a "
+                    help="instead of the serving benchmark: prefill / decode tokens/s of a layered hybrid design beside a "
                          "transformer of equal layer sizes (benchmarks/design_compare.py)")
+    ap.add_argument("--design", default="zadirax", choices=["zadirax", "pozalorn"], help="the design --design-compare measures")
+    ap.add_argument("--design-only", action="store_true", help="--design-compare without the transformer runs")
     ap.add_argument("--design-sizes", default="1024,1536", help="widths to compare (1024, 1536)")
     ap.add_argument("--design-prefill", type=int, default=2048)
     ap.add_argument("--design-batch", type=int, default=32)
@@ -367,7 +369,7 @@ def main():
         sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmarks"))
         import design_compare
         design_compare.main([int(x) for x in args.design_sizes.split(",")], args.design_prefill, args.design_batch,
-                            args.design_context)
+                            args.design_context, design=args.design, only_design=args.design_only)
         return
     if args.switch_interval_us > 0:
         sys.setswitchinterval(args.switch_interval_us * 1e-6)

@@ -1,7 +1,9 @@
-"""Prefill and decode throughput of the Zadirax design beside the closest transformer family at equal
-layer sizes (random weights, 4 layers each), through the engine's own step path.
+"""Prefill and decode throughput of a layered hybrid design (Zadirax, Pozalorn) beside the closest
+transformer family at equal layer sizes (random weights, the same number of layers), through the
+engine's own step path.
 
-    python bench.py --design-compare [--design-sizes 1024,1536] [--design-prefill 2048] [--design-batch 32]
+    python bench.py --design-compare [--design zadirax|pozalorn] [--design-sizes 1024,1536]
+                    [--design-prefill 2048] [--design-batch 32] [--design-context 512]
 
 Both models run teacher-forced steps (``LLMEngine.replay_step``: cache manager, step metadata, model
 forward and kernels; eager launches, nothing sampled):
@@ -72,26 +74,28 @@ def measure(model: str, overrides: dict | None, prefill: int, batch: int, contex
     return out
 
 
-SIZES = {
-    # width: (hybrid preset, transformer overrides at equal width / heads / feed-forward / vocabulary)
-    1024: ("zadirax-bench-1024", dict(hidden_size=1024, num_layers=4, num_heads=8, num_kv_heads=2, intermediate_size=4096,
-                                      vocab_size=32000, tie_embeddings=False)),
-    1536: ("zadirax-bench-1536", dict(hidden_size=1536, num_layers=4, num_heads=12, num_kv_heads=2, intermediate_size=8960,
-                                      vocab_size=32000, tie_embeddings=False)),
-}
+# transformer overrides at equal width / heads / feed-forward / vocabulary
+_QWEN = {1024: dict(hidden_size=1024, num_heads=8, num_kv_heads=2, intermediate_size=4096, vocab_size=32000, tie_embeddings=False),
+         1536: dict(hidden_size=1536, num_heads=12, num_kv_heads=2, intermediate_size=8960, vocab_size=32000, tie_embeddings=False)}
+# design -> (layers of its bench presets, "<design>-bench-<width>")
+DESIGNS = {"zadirax": 4, "pozalorn": 3}
 
 
-def main(sizes: list[int], prefill: int = 2048, batch: int = 32, context: int = 512) -> dict:
+def main(sizes: list[int], prefill: int = 2048, batch: int = 32, context: int = 512, design: str = "zadirax",
+         only_design: bool = False) -> dict:
+    layers = DESIGNS[design]
     summary = {}
     for w in sizes:
-        preset, ov = SIZES[w]
+        preset = f"{design}-bench-{w}"
         a = measure(preset, None, prefill, batch, context, 32000)
         print(json.dumps({"width": w, "model": preset, **a}), flush=True)
-        b = measure("qwen2.5-1.5b", ov, prefill, batch, context, 32000)
-        print(json.dumps({"width": w, "model": "qwen2 (4 layers, equal width)", **b}), flush=True)
+        if only_design:
+            continue
+        b = measure("qwen2.5-1.5b", dict(_QWEN[w], num_layers=layers), prefill, batch, context, 32000)
+        print(json.dumps({"width": w, "model": f"qwen2 ({layers} layers, equal width)", **b}), flush=True)
         summary[str(w)] = {"prefill_ratio": round(a["prefill_tok_s"] / b["prefill_tok_s"], 3),
                            "decode_ratio": round(a["decode_tok_s"] / b["decode_tok_s"], 3)}
-    line = {"metric": "Zadirax vs transformer at equal layer sizes, tokens/s ratio (4 layers, eager steps)",
+    line = {"metric": f"{design} vs transformer at equal layer sizes, tokens/s ratio ({layers} layers, eager steps)",
             "prefill_tokens": prefill, "decode_batch": batch, "decode_context": context, "ratios": summary}
     print(json.dumps(line), flush=True)
     return line

@@ -110,14 +110,18 @@ struct WindowArgs {
 };
 size_t window_attn_lds_bytes(const WindowArgs& a, int heads_per_block);
 bool window_attn_fits(const WindowArgs& a);   // sizes the kernels' LDS and register budgets take
-// q / k norm (qw, kw null: none; norm_all: one norm over the whole projection) + rotation + paged stores; q_out [T][H * D]
+// q / k norm (qw, kw null: none; norm_all: one norm over the whole projection) + rotation + paged stores; q_out [T][H * D];
+// vt: optional second, transposed bf16 copy of the values [pages][G][V][page]
 void launch_window_write(const WindowArgs& a, const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
-                         int64_t ldv, const float* qw, const float* kw, float eps, int norm_all, void* q_out,
+                         int64_t ldv, const float* qw, const float* kw, float eps, int norm_all, void* q_out, void* vt,
                          hipStream_t st);
 // pooled rows of the blocks this step's tokens complete
 void launch_window_pool(const WindowArgs& a, hipStream_t st);
 // out[t][h][:V] = softmax over (pooled blocks before the window, window tokens [, sink]) of scale q . key, times values
-void launch_window_attn(const WindowArgs& a, const void* q, float scale, void* out, hipStream_t st);
+// (vt: optional transposed bf16 copy of the values [pages][G][V][page] that window_write keeps; with it bf16
+// caches of head sizes in multiples of 8 up to 256 run the MFMA kernel)
+void launch_window_attn(const WindowArgs& a, const void* q, float scale, void* out, const void* vt, int num_pages,
+                        hipStream_t st);
 
 // Linear attention with decay over per-sequence state slots (linear_attn.hip).
 struct LinearAttnArgs {

@@ -17,6 +17,21 @@
 //               LDS as fp32; scores, running max / sum and the weighted value sum are fp32 FMA. A sink
 //               starts the running max at its logit and the running sum at 1. With turned values the
 //               normalised output is turned back by the query's position before it is stored.
+// window_attn, bf16 caches with head sizes in multiples of 8 up to 256: MFMA kernel. Rows are (token,
+//               query head of one key/value head) pairs of one sequence, 16 per wave, 4 independent waves
+//               per workgroup; keys in tiles of 32: first the pooled rows (two groups of 16, each lane
+//               addressing its own pooled row), then token tiles aligned to two whole pages.
+//                 S = Q K^T   v_mfma 16x16x32, Q fragments stationary, K fragments 16 B of a cached row
+//                 online softmax in fp32 (exp2 of log2(e)-scaled scores, per-lane partial row sums)
+//                 O += P V    P goes C-layout -> A-layout through a 16 x 32 bf16 tile in LDS; the B operand
+//                             needs eight consecutive KEYS of one value column per lane: for token tiles
+//                             window_write keeps a second, transposed copy of the values
+//                             ([page][G][column][16 keys]) so that is one 16-B load; for the (few) pooled
+//                             tiles the eight values are gathered from the pooled rows.
+//               Window, causal and pooled-block visibility are per-row masks on whole tiles, and tiles sit
+//               at fixed absolute key positions, so a row's sums do not depend on which rows share its wave.
+//               A sequence whose rows fit one wave (a decoded token) shares its tiles out over the
+//               workgroup's four waves, merged through LDS.
 // Every row of every kernel depends only on its own sequence's cache rows, in an order fixed by the
 // position, so results do not depend on how a prompt is cut or what else is in the batch.
 #include "common.h"
@@ -46,7 +61,8 @@ __global__ __launch_bounds__(256) void window_write_kernel(WindowArgs a, const v
                                                             const void* __restrict__ k, int64_t ldk,
                                                             const void* __restrict__ v, int64_t ldv,
                                                             const float* __restrict__ qw, const float* __restrict__ kw,
-                                                            float eps, int norm_all, void* __restrict__ q_out) {
+                                                            float eps, int norm_all, void* __restrict__ q_out,
+                                                            bf16_t* __restrict__ vt) {
   extern __shared__ float lds[];
   const int H = a.H, G = a.G, D = a.D, V = a.V;
   float* xs = lds;                    // [(H + G) * D] q heads then k heads
@@ -114,6 +130,7 @@ __global__ __launch_bounds__(256) void window_write_kernel(WindowArgs a, const v
       o = ldx(v, (int64_t)t * ldv + e, a.f32);
     }
     stx(a.vc, ((pg * G + g) * page + off) * V + i, a.f32, o);
+    if (vt != nullptr) vt[((pg * G + g) * V + i) * page + off] = f2bf(o);  // [page][G][column][key in page]
   }
 }
 
@@ -273,6 +290,282 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WindowArgs a, const vo
   }
 }
 
+
+// ---------------------------------------------------------------------------------- MFMA (bf16)
+__device__ __forceinline__ bf16x8 frag16(const bf16_t* rowp, int k, int K, bool valid) {
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (valid && k < K) {
+    const bf16_t* q = rowp + k;
+    if (k + 8 <= K && (reinterpret_cast<uintptr_t>(q) & 15) == 0) {
+      v = ld16(q);
+    } else {
+      uint32_t w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = (k + 2 * j < K) ? q[2 * j] : 0;
+        const uint32_t hi = (k + 2 * j + 1 < K) ? q[2 * j + 1] : 0;
+        w[j] = lo | (hi << 16);
+      }
+      v = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  }
+  return as_bf16x8(v);
+}
+
+// reductions over the 16 lanes that share l >> 4: rotations by 8, 4, 2, 1 inside the DPP row (VALU, no LDS)
+template <int CTRL>
+__device__ __forceinline__ float row_rot(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float group16_max(float v) {
+  v = fmaxf(v, row_rot<0x128>(v)); v = fmaxf(v, row_rot<0x124>(v));
+  v = fmaxf(v, row_rot<0x122>(v)); v = fmaxf(v, row_rot<0x121>(v));
+  return v;
+}
+__device__ __forceinline__ float group16_sum(float v) {
+  v += row_rot<0x128>(v); v += row_rot<0x124>(v); v += row_rot<0x122>(v); v += row_rot<0x121>(v);
+  return v;
+}
+
+// NCT: 16-column tiles of the value (V <= 16 NCT); NQF: 32-wide fragments of a query row (D <= 32 NQF).
+// D % 8 == 0 (host-checked): every key fragment is one unconditional 16-B load; a fragment past the row's
+// end or the value's last column is read from a clamped address: its partner (zero Q fragment) or its
+// output column (never stored) makes the value irrelevant, and cached values are always finite.
+constexpr int LG = 4;
+template <int NCT, int NQF>
+__global__ __launch_bounds__(256) void window_attn_mfma_kernel(WindowArgs a, const bf16_t* __restrict__ q,
+                                                                float scale_log2e, const bf16_t* __restrict__ vt,
+                                                                int num_pages, bf16_t* __restrict__ out) {
+  __shared__ __attribute__((aligned(16))) bf16_t pl[4][16][40];
+  __shared__ float mrg_m[4][16], mrg_l[4][16];
+  __shared__ float mrg_o[16][16 * NCT];  // split mode: the merged weighted values of the 16 rows
+  const int D = a.D, V = a.V, G = a.G, H = a.H, rep = H / G, g = blockIdx.y, P = a.pool;
+  int s = -1, tile = 0, base = 0;
+  for (int i = 0; i < a.S; ++i) {  // (sequence, 64-row tile) of this workgroup
+    const int nt = ((a.query_start[i + 1] - a.query_start[i]) * rep + 63) / 64;
+    if ((int)blockIdx.x < base + nt) { s = i; tile = blockIdx.x - base; break; }
+    base += nt;
+  }
+  if (s < 0) return;
+  const int wv = threadIdx.x >> 6, l = threadIdx.x & 63, lr = l & 15, lg = l >> 4;
+  const int t0 = a.query_start[s], ntok = a.query_start[s + 1] - t0;
+  const int pos0 = a.context_lens[s] - ntok;
+  const int nrows = ntok * rep;
+  const bool split = nrows <= 16;  // workgroup-uniform: one row tile, key tiles shared out over the four waves
+  const int row0 = split ? 0 : tile * 64 + wv * 16;
+  if (row0 >= nrows) return;
+  const bf16_t* kc = reinterpret_cast<const bf16_t*>(a.kc);
+  const bf16_t* kp = reinterpret_cast<const bf16_t*>(a.kp);
+  const bf16_t* vp = reinterpret_cast<const bf16_t*>(a.vp);
+  const int nqf = (D + 31) >> 5, nct = (V + 15) >> 4;
+  bf16x8 qf[NQF];  // stationary Q fragments: A operand, lane holds Q[row lr][32 kk + 8 lg ..]
+  {
+    const int r = row0 + lr;
+    const bool ok = r < nrows;
+    const bf16_t* qrow = q + ((int64_t)(t0 + (ok ? r / rep : 0)) * H + g * rep + (ok ? r % rep : 0)) * D;
+#pragma unroll
+    for (int kk = 0; kk < NQF; ++kk) qf[kk] = frag16(qrow, 32 * kk + 8 * lg, D, ok && kk < nqf);
+  }
+  // C-layout rows of this lane: row0 + 4 lg + i; what each sees: tokens [lo, hi], pooled blocks [0, nbv)
+  int hi[4], lo[4], nbv[4];
+  float m[4], lsum[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = row0 + 4 * lg + i;
+    const bool ok = r < nrows;
+    const int p = pos0 + (ok ? r / rep : 0);
+    hi[i] = ok ? p : -1;
+    lo[i] = p - a.window + 1;
+    nbv[i] = (ok && P > 0) ? max(0, lo[i]) / P : 0;
+    const bool sk = ok && a.sink != nullptr && (!split || wv == 0);  // the sink counts once
+    m[i] = sk ? a.sink[g * rep + r % rep] * 1.4426950408889634f : -INFINITY;
+    lsum[i] = (sk && lr == 0) ? 1.f : 0.f;
+  }
+  const int last = min(row0 + 15, nrows - 1);
+  const int pmin = pos0 + row0 / rep, pmax = pos0 + last / rep;  // wave-uniform
+  const int klo = max(0, pmin - a.window + 1);
+  const int nbmax = P > 0 ? max(0, pmax - a.window + 1) / P : 0;
+  const int ntp = (nbmax + 31) >> 5, jt0 = klo >> 5;
+  const int ntiles = ntp + (pmax >> 5) - jt0 + 1;
+  f32x4 O[NCT];
+#pragma unroll
+  for (int ct = 0; ct < NCT; ++ct) O[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int32_t* bt = a.block_tables + (int64_t)s * a.max_blocks;
+  for (int ti = split ? wv : 0; ti < ntiles; ti += split ? 4 : 1) {
+    const bool pooled = ti < ntp;  // wave-uniform
+    int kbase, pg0 = 0, pg1 = 0;
+    const bf16_t* k0p;
+    const bf16_t* k1p;
+    if (pooled) {
+      kbase = 32 * ti;
+      const int e0 = min(kbase + lr, nbmax - 1) * P + P - 1, e1 = min(kbase + 16 + lr, nbmax - 1) * P + P - 1;
+      const int q0 = min(max(bt[e0 >> 4], 0), num_pages - 1), q1 = min(max(bt[e1 >> 4], 0), num_pages - 1);
+      k0p = kp + (((int64_t)q0 * G + g) * a.npool + (e0 & 15) / P) * D;
+      k1p = kp + (((int64_t)q1 * G + g) * a.npool + (e1 & 15) / P) * D;
+    } else {
+      kbase = 32 * (jt0 + ti - ntp);
+      pg0 = bt[kbase >> 4];
+      pg1 = (kbase + 16 <= pmax) ? bt[(kbase >> 4) + 1] : pg0;
+      pg0 = min(max(pg0, 0), num_pages - 1);
+      pg1 = min(max(pg1, 0), num_pages - 1);
+      k0p = kc + (((int64_t)pg0 * G + g) * 16 + lr) * D;
+      k1p = kc + (((int64_t)pg1 * G + g) * 16 + lr) * D;
+    }
+    f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k0 = 0; k0 < NQF; k0 += LG) {
+      if (k0 < nqf) {  // wave-uniform
+        uint4 b0[LG], b1[LG];
+#pragma unroll
+        for (int u = 0; u < LG; ++u) {
+          const int off = min(32 * (k0 + u) + 8 * lg, D - 8);
+          b0[u] = ld16(k0p + off);
+          b1[u] = ld16(k1p + off);
+        }
+#pragma unroll
+        for (int u = 0; u < LG; ++u)
+          if (k0 + u < NQF) {
+            s0 = mfma16(qf[k0 + u], as_bf16x8(b0[u]), s0);
+            s1 = mfma16(qf[k0 + u], as_bf16x8(b1[u]), s1);
+          }
+      }
+    }
+    float al[4];
+    const int c0 = kbase + lr, c1 = kbase + 16 + lr;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool vis0 = pooled ? c0 < nbv[i] : (c0 >= lo[i] && c0 <= hi[i]);
+      const bool vis1 = pooled ? c1 < nbv[i] : (c1 >= lo[i] && c1 <= hi[i]);
+      const float v0 = vis0 ? s0[i] * scale_log2e : -INFINITY;
+      const float v1 = vis1 ? s1[i] * scale_log2e : -INFINITY;
+      const float mnew = fmaxf(m[i], group16_max(fmaxf(v0, v1)));
+      const float ms = (mnew == -INFINITY) ? 0.f : mnew;  // a row that has seen no key yet
+      al[i] = exp2f(m[i] - ms);
+      const float p0 = exp2f(v0 - ms), p1 = exp2f(v1 - ms);
+      lsum[i] = lsum[i] * al[i] + p0 + p1;
+      m[i] = mnew;
+      pl[wv][4 * lg + i][lr] = f2bf(p0);
+      pl[wv][4 * lg + i][16 + lr] = f2bf(p1);
+    }
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) O[ct][i] *= al[i];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's P tile is written (LDS is in order per wave)
+    const bf16x8 pf = as_bf16x8(*reinterpret_cast<const uint4*>(&pl[wv][lr][8 * lg]));
+    if (!pooled) {
+      const int pgs = (lg >> 1) ? pg1 : pg0;
+      const bf16_t* tp = vt + ((int64_t)pgs * G + g) * V * 16 + 8 * (lg & 1);
+#pragma unroll
+      for (int cb = 0; cb < NCT; cb += 2 * LG) {
+        if (cb < nct) {  // wave-uniform
+          uint4 b[2 * LG];
+#pragma unroll
+          for (int u = 0; u < 2 * LG; ++u) b[u] = ld16(tp + (int64_t)min(16 * (cb + u) + lr, V - 1) * 16);
+#pragma unroll
+          for (int u = 0; u < 2 * LG; ++u)
+            if (cb + u < NCT) O[cb + u] = mfma16(pf, as_bf16x8(b[u]), O[cb + u]);
+        }
+      }
+    } else {
+      // eight pooled rows per lane (keys kbase + 8 lg ..), one value column of each 16-column tile
+      int64_t ro[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int e1 = min(kbase + 8 * lg + e, nbmax - 1) * P + P - 1;
+        const int pq = min(max(bt[e1 >> 4], 0), num_pages - 1);
+        ro[e] = (((int64_t)pq * G + g) * a.npool + (e1 & 15) / P) * V;
+      }
+#pragma unroll
+      for (int ct = 0; ct < NCT; ++ct) {
+        if (ct < nct) {  // wave-uniform
+          const int col = min(16 * ct + lr, V - 1);
+          uint32_t w[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) w[j] = (uint32_t)vp[ro[2 * j] + col] | ((uint32_t)vp[ro[2 * j + 1] + col] << 16);
+          O[ct] = mfma16(pf, as_bf16x8(make_uint4(w[0], w[1], w[2], w[3])), O[ct]);
+        }
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // P tile read before the next tile overwrites it
+  }
+  if (split) {
+    float f[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float tot = group16_sum(lsum[i]);
+      if (lr == 0) { mrg_m[wv][4 * lg + i] = m[i]; mrg_l[wv][4 * lg + i] = tot; }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 4 * lg + i;
+      float M = mrg_m[0][r];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) M = fmaxf(M, mrg_m[w][r]);
+      const float Ms = (M == -INFINITY) ? 0.f : M;  // (rows past the sequence's last)
+      float L = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) L += mrg_l[w][r] * exp2f(mrg_m[w][r] - Ms);  // a wave that saw no key: l = 0, exp2(-inf) = 0
+      f[i] = exp2f(m[i] - Ms);
+      lsum[i] = L;                // the merged row sum (the same in every lane of the row)
+      m[i] = M;
+    }
+    for (int w = 0; w < 4; ++w) {  // waves add their scaled partials in turn
+      if (wv == w) {
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float* dst = &mrg_o[4 * lg + i][16 * ct + lr];
+            const float v = O[ct][i] * f[i];
+            *dst = (w == 0) ? v : *dst + v;
+          }
+      }
+      __syncthreads();
+    }
+    if (wv != 0) return;
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) O[ct][i] = mrg_o[4 * lg + i][16 * ct + lr];
+  }
+  const int vrot = a.v_freq != nullptr ? 2 * (V / 2) : 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float tot = split ? lsum[i] : group16_sum(lsum[i]);
+    const float inv = 1.f / tot;
+    const int r = row0 + 4 * lg + i;
+    const bool ok = r < nrows;
+    const float fp = -(float)(pos0 + (ok ? r / rep : 0));
+    bf16_t* orow = out + ((int64_t)(t0 + (ok ? r / rep : 0)) * H + g * rep + (ok ? r % rep : 0)) * V;
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct) {
+      const int col = 16 * ct + lr;
+      float y = O[ct][i] * inv;
+      if (vrot > 0) {  // turn the pair (even column, the next one) back by the row's position: the partner is lane l ^ 1
+        const float other = __shfl_xor(y, 1, 64);
+        if (col < vrot) {
+          const float ang = fp * a.v_freq[col >> 1];
+          const float cs = cosf(ang), sn = sinf(ang);
+          y = (col & 1) ? (y * cs + other * sn) : (y * cs - other * sn);
+        }
+      }
+      if (ok && ct < nct && col < V) orow[col] = f2bf(y);
+    }
+  }
+}
+
+template <int NCT, int NQF>
+void launch_window_mfma(const WindowArgs& a, const void* q, float scale, const void* vt, int num_pages, void* out,
+                        hipStream_t st) {
+  const int rep = a.H / a.G;
+  const int blocks = (a.T * rep + 63) / 64 + a.S;
+  hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF>), dim3(blocks, a.G), dim3(256), 0, st, a,
+                     reinterpret_cast<const bf16_t*>(q), scale * 1.4426950408889634f, reinterpret_cast<const bf16_t*>(vt),
+                     num_pages, reinterpret_cast<bf16_t*>(out));
+}
+
 int heads_per_block(const WindowArgs& a) {
   const int rep = a.H / a.G;
   int HC = rep < 8 ? rep : 8;
@@ -294,12 +587,12 @@ bool window_attn_fits(const WindowArgs& a) {
 }
 
 void launch_window_write(const WindowArgs& a, const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
-                         int64_t ldv, const float* qw, const float* kw, float eps, int norm_all, void* q_out,
+                         int64_t ldv, const float* qw, const float* kw, float eps, int norm_all, void* q_out, void* vt,
                          hipStream_t st) {
   if (a.T <= 0) return;
   const size_t lds = (size_t)((a.H + a.G) * a.D + a.H + a.G) * sizeof(float);
   hipLaunchKernelGGL(window_write_kernel, dim3(a.T), dim3(256), lds, st, a, q, ldq, k, ldk, v, ldv, qw, kw, eps, norm_all,
-                     q_out);
+                     q_out, reinterpret_cast<bf16_t*>(vt));
 }
 
 void launch_window_pool(const WindowArgs& a, hipStream_t st) {
@@ -307,8 +600,15 @@ void launch_window_pool(const WindowArgs& a, hipStream_t st) {
   hipLaunchKernelGGL(window_pool_kernel, dim3(a.T), dim3(256), 0, st, a);
 }
 
-void launch_window_attn(const WindowArgs& a, const void* q, float scale, void* out, hipStream_t st) {
+void launch_window_attn(const WindowArgs& a, const void* q, float scale, void* out, const void* vt, int num_pages,
+                        hipStream_t st) {
   if (a.T <= 0 || a.S <= 0) return;
+  if (!a.f32 && vt != nullptr && a.page == 16 && a.D % 8 == 0 && a.D >= 8 && a.D <= 256 && a.V <= 256) {
+    if (a.D <= 64 && a.V <= 64) launch_window_mfma<4, 2>(a, q, scale, vt, num_pages, out, st);
+    else if (a.D <= 128 && a.V <= 128) launch_window_mfma<8, 4>(a, q, scale, vt, num_pages, out, st);
+    else launch_window_mfma<16, 8>(a, q, scale, vt, num_pages, out, st);
+    return;
+  }
   const int HC = heads_per_block(a);
   const int rep = a.H / a.G;
   hipLaunchKernelGGL(window_attn_kernel, dim3(a.T, a.G, (rep + HC - 1) / HC), dim3(256), window_attn_lds_bytes(a, HC), st,

@@ -326,9 +326,18 @@ vgate::WindowArgs window_common(const Tensor& kc, const Tensor& vc, const OptT& 
   return a;
 }
 
+// the transposed bf16 value copy [pages, G, V, page] of a bf16 value cache [pages, G, page, V]
+void* window_vt(const OptT& vt, const Tensor& vc) {
+  if (!has(vt)) return nullptr;
+  TORCH_CHECK(vc.scalar_type() == torch::kBFloat16 && vt->is_cuda() && vt->scalar_type() == torch::kBFloat16 &&
+              vt->is_contiguous() && vt->dim() == 4 && vt->size(0) == vc.size(0) && vt->size(1) == vc.size(1) &&
+              vt->size(2) == vc.size(3) && vt->size(3) == vc.size(2), "window: vt bf16 [pages, G, V, page] beside a bf16 vc");
+  return vt->data_ptr();
+}
+
 void window_write(const Tensor& q, const Tensor& k, const Tensor& v, const OptT& qw, const OptT& kw, double eps,
                   bool norm_all, const Tensor& positions, const Tensor& slots, const Tensor& inv_freq, int64_t rot_dims,
-                  const OptT& v_freq, Tensor& kc, Tensor& vc, Tensor& q_out, int64_t H, int64_t G) {
+                  const OptT& v_freq, Tensor& kc, Tensor& vc, Tensor& q_out, int64_t H, int64_t G, const OptT& vt) {
   auto a = window_common(kc, vc, c10::nullopt, c10::nullopt, H, 0);
   TORCH_CHECK(G == a.G, "window_write: kv heads");
   const int64_t T = q.size(0);
@@ -348,9 +357,10 @@ void window_write(const Tensor& q, const Tensor& k, const Tensor& v, const OptT&
   TORCH_CHECK(has(qw) == has(kw), "window_write: q / k norm weights come together");
   const float* qwp = f32p(qw, "qw", norm_all ? H * a.D : a.D);
   const float* kwp = f32p(kw, "kw", norm_all ? G * a.D : a.D);
+  void* vtp = window_vt(vt, vc);
   c10::DeviceGuard guard(q.device());
   vgate::launch_window_write(a, q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), qwp, kwp,
-                             (float)eps, norm_all ? 1 : 0, q_out.data_ptr(), cur_stream());
+                             (float)eps, norm_all ? 1 : 0, q_out.data_ptr(), vtp, cur_stream());
 }
 
 void window_seq_meta(vgate::WindowArgs& a, const Tensor& block_tables, const Tensor& query_start) {
@@ -373,7 +383,7 @@ void window_pool(const Tensor& kc, const Tensor& vc, const OptT& kp, const OptT&
 
 void window_attn(const Tensor& q, const Tensor& kc, const Tensor& vc, const OptT& kp, const OptT& vp,
                  const Tensor& block_tables, const Tensor& context_lens, const Tensor& query_start, Tensor& out,
-                 double scale, int64_t H, int64_t window, int64_t pool, const OptT& sink, const OptT& v_freq) {
+                 double scale, int64_t H, int64_t window, int64_t pool, const OptT& sink, const OptT& v_freq, const OptT& vt) {
   auto a = window_common(kc, vc, kp, vp, H, pool);
   window_seq_meta(a, block_tables, query_start);
   a.context_lens = i32p(context_lens, "context_lens", a.S);
@@ -385,8 +395,9 @@ void window_attn(const Tensor& q, const Tensor& kc, const Tensor& vc, const OptT
   a.T = (int)T; a.window = (int)window;
   a.sink = f32p(sink, "sink", H);
   a.v_freq = f32p(v_freq, "v_freq", a.V / 2);
+  const void* vtp = window_vt(vt, vc);
   c10::DeviceGuard guard(q.device());
-  vgate::launch_window_attn(a, q.data_ptr(), (float)scale, out.data_ptr(), cur_stream());
+  vgate::launch_window_attn(a, q.data_ptr(), (float)scale, out.data_ptr(), vtp, (int)kc.size(0), cur_stream());
 }
 
 void linear_attn(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& g, const OptT& z, const OptT& head_decay,
@@ -496,9 +507,15 @@ void bind_seq(pybind11::module& m) {
         py::arg("x"), py::arg("y1"), py::arg("w"), py::arg("eps"), py::arg("out"), py::arg("s1") = 1.0,
         py::arg("y2") = py::none(), py::arg("s2") = 1.0, py::arg("act_out") = py::none(), py::arg("hist") = py::none(),
         py::arg("planes") = 0, py::arg("coef") = py::none(), py::arg("mix") = py::none());
-  m.def("window_write", &window_write, "q / k norm + rotation + paged key / value stores of window attention");
+  m.def("window_write", &window_write, "q / k norm + rotation + paged key / value stores of window attention", py::arg("q"),
+        py::arg("k"), py::arg("v"), py::arg("qw"), py::arg("kw"), py::arg("eps"), py::arg("norm_all"), py::arg("positions"),
+        py::arg("slots"), py::arg("inv_freq"), py::arg("rot_dims"), py::arg("v_freq"), py::arg("kc"), py::arg("vc"),
+        py::arg("q_out"), py::arg("H"), py::arg("G"), py::arg("vt") = py::none());
   m.def("window_pool", &window_pool, "mean key / value rows of the blocks a step completes");
-  m.def("window_attn", &window_attn, "sliding-window attention with pooled blocks and an optional sink");
+  m.def("window_attn", &window_attn, "sliding-window attention with pooled blocks and an optional sink", py::arg("q"),
+        py::arg("kc"), py::arg("vc"), py::arg("kp"), py::arg("vp"), py::arg("block_tables"), py::arg("context_lens"),
+        py::arg("query_start"), py::arg("out"), py::arg("scale"), py::arg("H"), py::arg("window"), py::arg("pool"),
+        py::arg("sink"), py::arg("v_freq"), py::arg("vt") = py::none());
   m.def("linear_attn", &linear_attn, "decayed linear attention recurrence over state slots + norm + gate");
   m.def("moe_route", &moe_route, "sigmoid router: corrected top-k choice, normalised uncorrected weights");
   m.def("moe_sort", &moe_sort, "counting sort of (token, choice) pairs by expert");

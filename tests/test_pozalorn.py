@@ -372,9 +372,10 @@ def _step_meta(lens_new, ctx, tables, d):
     return i32(pos), i32(slots), i32(qs), i32(ctx)
 
 
-def _run_window(d, dt, q, k, v, H, G, size, pool, sink, turn, tables, steps):
+def _run_window(d, dt, q, k, v, H, G, size, pool, sink, turn, tables, steps, transposed=False):
     """Feed sequences through window_write / window_pool / window_attn in the given steps
-    (``steps``: list of per-sequence new-token counts); returns each sequence's outputs [T, H * V]."""
+    (``steps``: list of per-sequence new-token counts); returns each sequence's outputs [T, H * V].
+    ``transposed``: keep the transposed value copy, which selects the MFMA kernel (GPU, bf16)."""
     from vgate.ops import seq
     S, D, V = len(q), q[0].shape[1] // H, v[0].shape[1] // G
     pages = int(max(max(t) for t in tables)) + 1
@@ -383,6 +384,7 @@ def _run_window(d, dt, q, k, v, H, G, size, pool, sink, turn, tables, steps):
     vc = torch.full((pages, G, 16, V), -9.0, dtype=dt, device=d)
     kp = torch.full((pages, G, npool, D), 9.0, dtype=dt, device=d) if pool else None
     vp = torch.full((pages, G, npool, V), -9.0, dtype=dt, device=d) if pool else None
+    vt = torch.full((pages, G, V, 16), -9.0, dtype=dt, device=d) if transposed else None
     bt = torch.zeros(S, max(len(t) for t in tables), dtype=torch.int32)
     for s, t in enumerate(tables):
         bt[s, : len(t)] = torch.tensor(t, dtype=torch.int32)
@@ -397,11 +399,11 @@ def _run_window(d, dt, q, k, v, H, G, size, pool, sink, turn, tables, steps):
         cat = lambda xs: torch.cat([xs[s][done[s]: ctx[s]] for s in range(S)]).to(d, dt)  # noqa: E731
         T = int(qs[-1])
         qo = torch.zeros(T, H * D, dtype=dt, device=d)
-        seq.window_write(cat(q), cat(k), cat(v), None, None, 1e-6, False, pos, slots, none, 0, vf, kc, vc, qo, H, G)
+        seq.window_write(cat(q), cat(k), cat(v), None, None, 1e-6, False, pos, slots, none, 0, vf, kc, vc, qo, H, G, vt=vt)
         if pool:
             seq.window_pool(kc, vc, kp, vp, pos, bt, qs, pool)
         o = torch.zeros(T, H * V, dtype=dt, device=d)
-        seq.window_attn(qo, kc, vc, kp, vp, bt, cl, qs, o, 0.5, H, size, pool, sink, vf)
+        seq.window_attn(qo, kc, vc, kp, vp, bt, cl, qs, o, 0.5, H, size, pool, sink, vf, vt=vt)
         for s in range(S):
             outs[s].append(o[int(qs[s]): int(qs[s + 1])].float().cpu())
         done = ctx
@@ -459,8 +461,9 @@ def test_window_attention_edges(device, f32, size, pool):
         want = _want_window(q, k, v, H, G, size, pool, sk, turn)
         skd = sk.to(d) if use_sink else None
         for steps in ([[T]], [[61], [2], [35], [1], [1], [50]], [[T - 40]] + [[1]] * 40):
-            got = _run_window(d, dt, [q], [k], [v], H, G, size, pool, skd, turn, tables, steps)[0]
-            assert rel(got, want) < (3e-5 if f32 else 2e-2), (use_sink, turn, len(steps))
+            for mfma in ([False, True] if device == "cuda" and not f32 else [False]):
+                got = _run_window(d, dt, [q], [k], [v], H, G, size, pool, skd, turn, tables, steps, transposed=mfma)[0]
+                assert rel(got, want) < (3e-5 if f32 else 2e-2), (use_sink, turn, len(steps), mfma)
         # the crafted keys matter: one more or one fewer key in the window moves the answer
         # (with pool 1 every earlier token is seen either way, as itself or as its own block)
         if pool != 1:
@@ -484,6 +487,10 @@ def test_window_attention_batch_and_page_reuse(device):
     # b again on a's pages, from position 0
     got = _run_window(d, torch.float32, [qb], [kb], [vb], H, G, 10, 4, None, True, [[3, 1, 4]], [[20], [17]])
     assert rel(got[0], wb) < 3e-5
+    if device == "cuda":   # the MFMA kernel: rows of two sequences, of several tokens and of one
+        got = _run_window(d, torch.bfloat16, [qa, qb], [ka, kb], [va, vb], H, G, 10, 4, None, True,
+                          [[3, 1, 4, 0, 2], [6, 5, 7]], [[30, 1], [2, 30], [38, 6]], transposed=True)
+        assert rel(got[0], wa) < 2e-2 and rel(got[1], wb) < 2e-2
 
 
 @pytest.mark.parametrize("device", DEVICES)

@@ -34,6 +34,8 @@ from vgate.ops import seq
 # through the row-major GEMM. "0" sends everything through the row-major one.
 USE_PACKED = os.environ.get("VGATE_HYBRID_PACKED", "1") == "1"
 PACKED_MIN_K = 512
+# bf16 window attention on the MFMA kernel (keeps a transposed copy of the values); "0": the FMA kernel
+USE_WINDOW_MFMA = os.environ.get("VGATE_WINDOW_MFMA", "1") == "1"
 
 
 class Proj:
@@ -299,27 +301,33 @@ class WindowAttention:
         dt = torch.float32 if self.f32 else torch.bfloat16
         npool = self.pooled_per_page(block_size)
         z = lambda rows, d: torch.zeros(num_blocks, self.G, rows, d, dtype=dt, device=device)  # noqa: E731
+        # bf16 on the GPU: a second, transposed copy of the values for the MFMA kernel's weighted sum
+        vt = torch.zeros(num_blocks, self.G, self.V, block_size, dtype=dt, device=device) if self._transposed(device) else None
         return (z(block_size, self.D), z(block_size, self.V),
-                z(npool, self.D) if npool else None, z(npool, self.V) if npool else None)
+                z(npool, self.D) if npool else None, z(npool, self.V) if npool else None, vt)
+
+    def _transposed(self, device) -> bool:
+        return not self.f32 and torch.device(device).type == "cuda" and USE_WINDOW_MFMA
 
     def page_bytes(self, block_size: int) -> int:
-        return (block_size + self.pooled_per_page(block_size)) * self.G * (self.D + self.V) * (4 if self.f32 else 2)
+        n = (block_size + self.pooled_per_page(block_size)) * self.G * (self.D + self.V) * (4 if self.f32 else 2)
+        return n + (0 if self.f32 else block_size * self.G * self.V * 2)
 
     def nbytes(self) -> int:
         return self.o.nbytes()
 
     def forward(self, h, P, cols, sv, cache) -> torch.Tensor:
         T = h.shape[0]
-        kc, vc, kp, vp = cache
+        kc, vc, kp, vp, vt = cache
         q = torch.empty(T, self.H * self.D, dtype=h.dtype, device=h.device)
         seq.window_write(cols(P, "q"), cols(P, "k"), cols(P, "v"), self.qw, self.kw, self.eps, self.qk_norm == "all",
-                         sv.positions, sv.slots, self.inv_freq, self.rot_dims, self.v_freq, kc, vc, q, self.H, self.G)
+                         sv.positions, sv.slots, self.inv_freq, self.rot_dims, self.v_freq, kc, vc, q, self.H, self.G, vt=vt)
         if self.pool:
             seq.window_pool(kc, vc, kp, vp, sv.positions, sv.block_tables, sv.query_start, self.pool,
                             num_seqs=sv.num_seqs or None)
         o = torch.empty(T, self.H * self.V, dtype=h.dtype, device=h.device)
         seq.window_attn(q, kc, vc, kp, vp, sv.block_tables, sv.context_lens, sv.query_start, o, self.scale, self.H,
-                        self.window, self.pool, self.sink, self.v_freq, num_seqs=sv.num_seqs or None)
+                        self.window, self.pool, self.sink, self.v_freq, num_seqs=sv.num_seqs or None, vt=vt)
         return self.o(o, out_f32=True)
 
 

@@ -346,15 +346,17 @@ def _rope_pairs_heads(x: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor
 
 
 def window_write(q, k, v, qw, kw, eps: float, norm_all: bool, positions, slots, inv_freq, rot_dims: int, v_freq,
-                 kc, vc, q_out, H: int, G: int) -> None:
+                 kc, vc, q_out, H: int, G: int, vt=None) -> None:
     """Prepare one step's queries, keys and values of a window-attention layer.
     q [T, H * D], k [T, G * D], v [T, G * V] (biases already added). Query / key RMS norm (``qw`` / ``kw``
     None: none; ``norm_all``: over the whole projection with a [heads * D] weight, else per head with a
     [D] weight), rotation of the first ``rot_dims`` entries of every head, values turned over all of V
     by ``v_freq`` if given. q goes to ``q_out``; keys and values to the paged caches
-    kc [pages, G, page, D] / vc [pages, G, page, V] at the tokens' slots (slot < 0: padding row)."""
+    kc [pages, G, page, D] / vc [pages, G, page, V] at the tokens' slots (slot < 0: padding row).
+    ``vt`` (GPU, bf16): a second copy of the values laid out [pages, G, V, page], the operand layout of
+    the MFMA attention kernel's weighted sum."""
     if q.is_cuda:
-        _C().window_write(q, k, v, qw, kw, eps, norm_all, positions, slots, inv_freq, rot_dims, v_freq, kc, vc, q_out, H, G)
+        _C().window_write(q, k, v, qw, kw, eps, norm_all, positions, slots, inv_freq, rot_dims, v_freq, kc, vc, q_out, H, G, vt)
         return
     T = q.shape[0]
     D, V, page = kc.shape[3], vc.shape[3], kc.shape[2]
@@ -405,14 +407,15 @@ def window_pool(kc, vc, kp, vp, positions, block_tables, query_start, pool: int,
 
 
 def window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out, scale: float, H: int, window: int,
-                pool: int, sink, v_freq, num_seqs: int | None = None) -> None:
+                pool: int, sink, v_freq, num_seqs: int | None = None, vt=None) -> None:
     """out[t, h] = sum_j p_j value_j over the keys position i of token t sees: the tokens j with
     0 <= i - j < window and, with ``pool`` = P > 0, the pooled row of every block b with
     b P + P - 1 <= i - window; p = softmax(scale q . key) over both kinds together, with exp(sink[h]) added
     to the denominator if ``sink`` is given. With ``v_freq`` the result is turned back by -i over all of V.
-    Query head h reads key/value head h / (H / G)."""
+    Query head h reads key/value head h / (H / G). With ``vt`` (see :func:`window_write`) bf16 caches run
+    the MFMA kernel."""
     if q.is_cuda:
-        _C().window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out, scale, H, window, pool, sink, v_freq)
+        _C().window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out, scale, H, window, pool, sink, v_freq, vt)
         return
     G, page, D, V = kc.shape[1], kc.shape[2], kc.shape[3], vc.shape[3]
     rep = H // G
