@@ -12,6 +12,12 @@
 //          while the current one computes. A sequence's tokens of the step run in order from the slot's
 //          state; a portion that starts at position 0 starts from zero, so a reused slot needs no clearing.
 //   finish token parallel: norm, norm weight, output gate, store in the activation dtype.
+// Long steps (a prompt portion of hundreds of tokens) run the scan over chunks of CH tokens in parallel:
+//   local   every chunk from a zero state: its local state L_c and the product A_c of its decays
+//   carry   per sequence, chunk after chunk: I_0 = slot state, I_(c+1) = diag(A_c) I_c + L_c (the same
+//           recurrence taken CH tokens at a time, all fp32); the slot receives the last one
+//   output  every chunk again from its true initial state I_c, now writing o
+// Twice the arithmetic, but a lone sequence's dependent chain is CH tokens long instead of the whole portion.
 #include "common.h"
 #include "seq_launchers.h"
 
@@ -49,28 +55,57 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(LinearAttnArgs p, floa
 }
 
 // lane = 8 * q + c: key group q of 8 (keys [q dq, (q + 1) dq) with dq = ceil(D / 8) <= DQ), value column c0 + c
-template <int DQ, int TC>
+// MODE 0: a sequence's whole portion from its slot. MODE 1 / 2: one chunk of CH tokens per blockIdx.x (chunks
+// of all sequences numbered in order), 1 = from zero, writes the chunk's local state and decay product;
+// 2 = from cstate[chunk], writes the outputs.
+enum { SCAN_WHOLE = 0, SCAN_LOCAL = 1, SCAN_OUTPUT = 2 };
+
+__device__ __forceinline__ bool locate_chunk(const LinearAttnArgs& p, int CH, int bx, int& s, int& t0, int& t1) {
+  int base = 0;
+  for (int i = 0; i < p.S; ++i) {
+    const int a = p.query_start[i], b = p.query_start[i + 1];
+    const int nc = (p.state_slots[i] < 0 || b <= a) ? 0 : (b - a + CH - 1) / CH;
+    if (bx < base + nc) {
+      s = i; t0 = a + (bx - base) * CH; t1 = min(b, t0 + CH);
+      return true;
+    }
+    base += nc;
+  }
+  return false;
+}
+
+template <int DQ, int TC, int MODE>
 __global__ __launch_bounds__(64) void linear_scan_kernel(LinearAttnArgs p, const float4* __restrict__ vec,
-                                                          const float* __restrict__ vals, float* __restrict__ oraw) {
+                                                          const float* __restrict__ vals, float* __restrict__ oraw,
+                                                          int CH, float* __restrict__ cstate, float* __restrict__ cdecay) {
   constexpr int QV = DQ + 1;             // padded group stride: the groups' broadcast reads hit different banks
   constexpr int NE = (8 * DQ + 63) / 64;  // channels a lane stages per token
   __shared__ float4 lv[2][TC][8 * QV];
   __shared__ float lvv[2][TC][8];
-  const int s = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * 8;
-  const int slot = p.state_slots[s];
-  const int t0 = p.query_start[s], t1 = p.query_start[s + 1];
-  if (slot < 0 || t1 <= t0) return;
+  const int h = blockIdx.y, c0 = blockIdx.z * 8;
+  int s = blockIdx.x, t0, t1;
+  if (MODE == SCAN_WHOLE) {
+    t0 = p.query_start[s]; t1 = p.query_start[s + 1];
+    if (p.state_slots[s] < 0 || t1 <= t0) return;
+  } else if (!locate_chunk(p, CH, blockIdx.x, s, t0, t1)) {
+    return;
+  }
   const int D = p.D, V = p.V, lane = threadIdx.x;
   const int q = lane >> 3, c = c0 + (lane & 7);
   const int dq = (D + 7) >> 3;
   const int k0 = q * dq;
   const bool con = c < V;
-  const int pos0 = p.context_lens[s] - (t1 - t0);
-  float* sp = p.state + ((int64_t)slot * p.H + h) * D * V;
-  float S[DQ];
+  // where this block's state starts from and goes to
+  float* sp = MODE == SCAN_WHOLE ? p.state + ((int64_t)p.state_slots[s] * p.H + h) * D * V
+                                 : cstate + ((int64_t)blockIdx.x * p.H + h) * D * V;
+  const bool from_zero = MODE == SCAN_LOCAL ||
+                         (MODE == SCAN_WHOLE && p.context_lens[s] - (t1 - t0) <= 0);
+  float S[DQ], A[MODE == SCAN_LOCAL ? DQ : 1];
 #pragma unroll
-  for (int j = 0; j < DQ; ++j)
-    S[j] = (con && j < dq && k0 + j < D && pos0 > 0) ? sp[(int64_t)(k0 + j) * V + c] : 0.f;
+  for (int j = 0; j < DQ; ++j) {
+    S[j] = (con && j < dq && k0 + j < D && !from_zero) ? sp[(int64_t)(k0 + j) * V + c] : 0.f;
+    if (MODE == SCAN_LOCAL) A[j] = 1.f;
+  }
   float4 pv[TC][NE];
   float pvv[(TC * 8 + 63) / 64];
   auto fetch = [&](int tb) {
@@ -119,12 +154,15 @@ __global__ __launch_bounds__(64) void linear_scan_kernel(LinearAttnArgs p, const
       for (int j = 0; j < DQ; ++j) {
         const float4 x = tv[j];  // {a, k, q}
         S[j] = fmaf(x.y, vv, x.x * S[j]);
-        o = fmaf(x.z, S[j], o);
+        if (MODE == SCAN_LOCAL) A[j] *= x.x;
+        else o = fmaf(x.z, S[j], o);
       }
-      o += xor8(o);
-      o += xor16(o);
-      o += xor32(o);
-      if (con && q == 0) oraw[((int64_t)(tb + i) * p.H + h) * V + c] = o;
+      if (MODE != SCAN_LOCAL) {
+        o += xor8(o);
+        o += xor16(o);
+        o += xor32(o);
+        if (con && q == 0) oraw[((int64_t)(tb + i) * p.H + h) * V + c] = o;
+      }
     }
     if (more) {
       put(buf ^ 1);
@@ -132,9 +170,45 @@ __global__ __launch_bounds__(64) void linear_scan_kernel(LinearAttnArgs p, const
       buf ^= 1;
     }
   }
+  if (MODE == SCAN_OUTPUT) return;
 #pragma unroll
   for (int j = 0; j < DQ; ++j)
     if (con && j < dq && k0 + j < D) sp[(int64_t)(k0 + j) * V + c] = S[j];
+  if (MODE == SCAN_LOCAL && blockIdx.z == 0 && (lane & 7) == 0) {
+#pragma unroll
+    for (int j = 0; j < DQ; ++j)
+      if (j < dq && k0 + j < D) cdecay[((int64_t)blockIdx.x * p.H + h) * D + k0 + j] = A[MODE == SCAN_LOCAL ? j : 0];
+  }
+}
+
+// one workgroup per (sequence, head): I_0 = slot state (zero at position 0), I_(c+1) = diag(A_c) I_c + L_c;
+// cstate[c] becomes I_c, the slot the state after the last chunk
+__global__ __launch_bounds__(256) void linear_carry_kernel(LinearAttnArgs p, int CH, float* __restrict__ cstate,
+                                                            const float* __restrict__ cdecay) {
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int slot = p.state_slots[s];
+  const int t0 = p.query_start[s], t1 = p.query_start[s + 1];
+  if (slot < 0 || t1 <= t0) return;
+  int base = 0;
+  for (int i = 0; i < s; ++i) {
+    const int a = p.query_start[i], b = p.query_start[i + 1];
+    base += (p.state_slots[i] < 0 || b <= a) ? 0 : (b - a + CH - 1) / CH;
+  }
+  const int nc = (t1 - t0 + CH - 1) / CH;
+  const int D = p.D, V = p.V;
+  const bool from_zero = p.context_lens[s] - (t1 - t0) <= 0;
+  float* sp = p.state + ((int64_t)slot * p.H + h) * D * V;
+  for (int e = threadIdx.x; e < D * V; e += blockDim.x) {
+    const int k = e / V;
+    float cur = from_zero ? 0.f : sp[e];
+    for (int c = 0; c < nc; ++c) {
+      float* cs = cstate + ((int64_t)(base + c) * p.H + h) * D * V + e;
+      const float loc = *cs;
+      *cs = cur;
+      cur = fmaf(cdecay[((int64_t)(base + c) * p.H + h) * D + k], cur, loc);
+    }
+    sp[e] = cur;
+  }
 }
 
 // one workgroup per token; waves take heads in turn
@@ -169,21 +243,51 @@ __global__ __launch_bounds__(256) void linear_finish_kernel(LinearAttnArgs p, co
   }
 }
 
+template <int DQ, int TC>
+void launch_scan(const LinearAttnArgs& a, int T, const float4* vec, const float* vals, float* oraw, int CH, float* cstate,
+                 float* cdecay, hipStream_t st) {
+  const int cols = (a.V + 7) / 8;
+  if (CH <= 0) {
+    hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, SCAN_WHOLE>), dim3(a.S, a.H, cols), dim3(64), 0, st, a, vec, vals, oraw,
+                       0, nullptr, nullptr);
+    return;
+  }
+  const int chunks = linear_attn_chunks(T, a.S, CH);
+  hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, SCAN_LOCAL>), dim3(chunks, a.H, cols), dim3(64), 0, st, a, vec, vals, oraw,
+                     CH, cstate, cdecay);
+  hipLaunchKernelGGL(linear_carry_kernel, dim3(a.S, a.H), dim3(256), 0, st, a, CH, cstate, cdecay);
+  hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, SCAN_OUTPUT>), dim3(chunks, a.H, cols), dim3(64), 0, st, a, vec, vals, oraw,
+                     CH, cstate, cdecay);
+}
+
 }  // namespace
 
-// scratch: T * H * (4 D + 2 V) floats ({a, k, q, -} per key channel, the values, the raw outputs)
+int linear_attn_chunk_size(int T, int S) {
+  // steps of a few tokens per sequence (decoding, short portions): one pass per sequence; long ones: chunks
+  return T >= 256 && T >= 64 * S ? 64 : 0;
+}
+int linear_attn_chunks(int T, int S, int CH) { return CH > 0 ? T / CH + S : 0; }
+size_t linear_attn_scratch_floats(int T, int S, int H, int D, int V) {
+  const int CH = linear_attn_chunk_size(T, S);
+  return (size_t)T * H * (4 * D + 2 * V) + (size_t)linear_attn_chunks(T, S, CH) * H * D * (V + 1);
+}
+
+// scratch: linear_attn_scratch_floats(): {a, k, q, -} per key channel, the values, the raw outputs, and for
+// chunked steps every chunk's state and decay product
 void launch_linear_attn(const LinearAttnArgs& a, int T, float* scratch, hipStream_t st) {
   if (a.S <= 0 || a.H <= 0 || T <= 0) return;
   const int64_t nk = (int64_t)T * a.H * a.D, nv = (int64_t)T * a.H * a.V;
   float4* vec = reinterpret_cast<float4*>(scratch);
   float* vals = scratch + 4 * nk;
   float* oraw = vals + nv;
+  const int CH = linear_attn_chunk_size(T, a.S);
+  float* cstate = oraw + nv;
+  float* cdecay = cstate + (size_t)linear_attn_chunks(T, a.S, CH) * a.H * a.D * a.V;
   hipLaunchKernelGGL(linear_prep_kernel, dim3(T), dim3(256), 0, st, a, vec, vals);
-  const dim3 grid(a.S, a.H, (a.V + 7) / 8);
-  if (a.D <= 32) hipLaunchKernelGGL((linear_scan_kernel<4, 8>), grid, dim3(64), 0, st, a, vec, vals, oraw);
-  else if (a.D <= 64) hipLaunchKernelGGL((linear_scan_kernel<8, 8>), grid, dim3(64), 0, st, a, vec, vals, oraw);
-  else if (a.D <= 128) hipLaunchKernelGGL((linear_scan_kernel<16, 8>), grid, dim3(64), 0, st, a, vec, vals, oraw);
-  else hipLaunchKernelGGL((linear_scan_kernel<32, 4>), grid, dim3(64), 0, st, a, vec, vals, oraw);
+  if (a.D <= 32) launch_scan<4, 8>(a, T, vec, vals, oraw, CH, cstate, cdecay, st);
+  else if (a.D <= 64) launch_scan<8, 8>(a, T, vec, vals, oraw, CH, cstate, cdecay, st);
+  else if (a.D <= 128) launch_scan<16, 8>(a, T, vec, vals, oraw, CH, cstate, cdecay, st);
+  else launch_scan<32, 4>(a, T, vec, vals, oraw, CH, cstate, cdecay, st);
   hipLaunchKernelGGL(linear_finish_kernel, dim3(T), dim3(256), 0, st, a, oraw);
 }
 

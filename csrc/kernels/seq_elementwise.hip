@@ -78,6 +78,26 @@ __global__ __launch_bounds__(256) void cast_rows_kernel(const float* __restrict_
   if (i < n) y[i] = f2bf(x[i]);
 }
 
+// out[t][j] = act(gu[t][j]) * gu[t][n + j] for a stacked [gate; up] projection (bf16), 8 columns per thread
+__global__ __launch_bounds__(256) void glu_rows_kernel(const bf16_t* __restrict__ gu, int64_t ldg, bf16_t* __restrict__ out,
+                                                        int64_t ldo, int n, int act, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int per = n / 8;
+  const int64_t t = i / per;
+  const int j = (int)(i % per) * 8;
+  float g[8], u[8];
+  unpack8(ld16(gu + t * ldg + j), g);
+  unpack8(ld16(gu + t * ldg + n + j), u);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float x = g[e];
+    const float a = act == 4 ? 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x))) : x * sigm(x);
+    g[e] = a * u[e];
+  }
+  *reinterpret_cast<uint4*>(out + t * ldo + j) = pack8(g);
+}
+
 // one workgroup per token; every element is read and written by the same thread, so out may be x and
 // mix may be x
 __global__ __launch_bounds__(256) void post_norm_add_kernel(PostNormArgs a) {
@@ -180,6 +200,13 @@ void launch_cast_rows(const float* x, void* y, int T, int n, hipStream_t st) {
   if (tot <= 0) return;
   hipLaunchKernelGGL(cast_rows_kernel, dim3((unsigned)((tot + 255) / 256)), dim3(256), 0, st, x,
                      reinterpret_cast<bf16_t*>(y), tot);
+}
+
+void launch_glu_rows(const void* gu, int64_t ldg, void* out, int64_t ldo, int T, int n, int act, hipStream_t st) {
+  const int64_t total = (int64_t)T * (n / 8);
+  if (total <= 0) return;
+  hipLaunchKernelGGL(glu_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                     reinterpret_cast<const bf16_t*>(gu), ldg, reinterpret_cast<bf16_t*>(out), ldo, n, act, total);
 }
 
 void launch_post_norm_add(const PostNormArgs& a, hipStream_t st) {

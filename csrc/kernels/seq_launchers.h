@@ -43,6 +43,8 @@ void launch_gated_residual(float* x, const void* y1, const void* g1, int64_t ldg
 
 // y = x rounded to the activation dtype (bf16), rows of n
 void launch_cast_rows(const float* x, void* y, int T, int n, hipStream_t st);
+// out[t][j] = act(gu[t][j]) * gu[t][n + j], j < n (bf16 rows, n % 8 == 0, 16-B aligned); act 1 silu, 4 gelu_tanh
+void launch_glu_rows(const void* gu, int64_t ldg, void* out, int64_t ldo, int T, int n, int act, hipStream_t st);
 // out = x + u * rsqrt(mean(u^2) + eps) * w, u = s1 y1 [+ s2 y2] (fp32; out may alias x). With hist
 // ([planes][T][W] fp32, plane stride hist_ps, whose last used plane is out): mix = sum_j coef[j] hist[j].
 // act_out (bf16): a copy of mix, or of out without hist.
@@ -137,7 +139,12 @@ struct LinearAttnArgs {
   void* out = nullptr; int64_t ldo = 0;
   int S = 0, H = 0, D = 0, V = 0, f32 = 0;
 };
-// T rows; scratch: T * H * (4 D + 2 V) floats, 16-B aligned
+// tokens per chunk a step of T rows over S sequences is scanned in (0: every sequence in one pass), the
+// chunks such a step has at most, and the scratch floats it needs
+int linear_attn_chunk_size(int T, int S);
+int linear_attn_chunks(int T, int S, int CH);
+size_t linear_attn_scratch_floats(int T, int S, int H, int D, int V);
+// T rows; scratch: linear_attn_scratch_floats() floats, 16-B aligned
 void launch_linear_attn(const LinearAttnArgs& a, int T, float* scratch, hipStream_t st);
 
 // idx, wts [T][top]: the `top` largest of sigmoid(z) + corr; wts = sigmoid(z) of the chosen / their sum

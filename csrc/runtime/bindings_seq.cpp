@@ -261,6 +261,20 @@ void cast_rows(const Tensor& x, Tensor& y) {
   vgate::launch_cast_rows(x.data_ptr<float>(), y.data_ptr(), (int)y.size(0), (int)y.size(1), cur_stream());
 }
 
+void glu_rows(const Tensor& gu, Tensor& out, int64_t act) {
+  TORCH_CHECK(gu.is_cuda() && gu.scalar_type() == torch::kBFloat16 && gu.dim() == 2 && gu.stride(1) == 1, "glu_rows: gu bf16 [T, 2 n]");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == torch::kBFloat16 && out.dim() == 2 && out.stride(1) == 1 &&
+              out.size(0) <= gu.size(0) && gu.size(1) == 2 * out.size(1), "glu_rows: out bf16 [<= T, n]");
+  const int64_t n = out.size(1);
+  TORCH_CHECK(n % 8 == 0 && gu.stride(0) % 8 == 0 && out.stride(0) % 8 == 0 &&
+              (reinterpret_cast<uintptr_t>(gu.data_ptr()) & 15) == 0 && (reinterpret_cast<uintptr_t>(out.data_ptr()) & 15) == 0,
+              "glu_rows: rows of whole 16-B pieces");
+  TORCH_CHECK(act == 1 || act == 4, "glu_rows: act 1 (silu) or 4 (gelu_tanh)");
+  c10::DeviceGuard guard(gu.device());
+  vgate::launch_glu_rows(gu.data_ptr(), gu.stride(0), out.data_ptr(), out.stride(0), (int)out.size(0), (int)n, (int)act,
+                         cur_stream());
+}
+
 void post_norm_add(const Tensor& x, const Tensor& y1, const Tensor& w, double eps, Tensor& out, double s1, const OptT& y2,
                    double s2, const OptT& act_out, const OptT& hist, int64_t planes, const OptT& coef, const OptT& mix) {
   auto f32_2d = [](const Tensor& t, const char* name) {
@@ -436,7 +450,8 @@ void linear_attn(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor
   p.context_lens = i32p(context_lens, "context_lens", p.S);
   p.query_start = i32p(query_start, "query_start", p.S + 1);
   TORCH_CHECK(scratch.is_cuda() && scratch.scalar_type() == torch::kFloat32 && scratch.is_contiguous() &&
-              scratch.numel() >= T * (4 * HD + 2 * HV), "linear_attn: scratch fp32 with T * H * (4 D + 2 V) elements");
+              (size_t)scratch.numel() >= vgate::linear_attn_scratch_floats((int)T, p.S, p.H, p.D, p.V),
+              "linear_attn: scratch fp32 with linear_attn_scratch(T, S, H, D, V) elements");
   TORCH_CHECK((reinterpret_cast<uintptr_t>(scratch.data_ptr()) & 15) == 0, "linear_attn: scratch must be 16-B aligned");
   c10::DeviceGuard guard(q.device());
   vgate::launch_linear_attn(p, (int)T, scratch.data_ptr<float>(), cur_stream());
@@ -503,6 +518,7 @@ void bind_seq(pybind11::module& m) {
         py::arg("scale"), py::arg("H"), py::arg("rank"), py::arg("rot"), py::arg("cache_t") = py::none());
   m.def("delta_rule", &delta_rule, "generalized delta rule recurrence over state slots + head norm + gate");
   m.def("cast_rows", &cast_rows, "fp32 rows rounded to bf16");
+  m.def("glu_rows", &glu_rows, "out = act(gate) * up over a stacked [gate; up] projection");
   m.def("post_norm_add", &post_norm_add, "out = x + rmsnorm(s1 y1 + s2 y2) * w, optional depth average and bf16 copy",
         py::arg("x"), py::arg("y1"), py::arg("w"), py::arg("eps"), py::arg("out"), py::arg("s1") = 1.0,
         py::arg("y2") = py::none(), py::arg("s2") = 1.0, py::arg("act_out") = py::none(), py::arg("hist") = py::none(),
@@ -516,6 +532,9 @@ void bind_seq(pybind11::module& m) {
         py::arg("kc"), py::arg("vc"), py::arg("kp"), py::arg("vp"), py::arg("block_tables"), py::arg("context_lens"),
         py::arg("query_start"), py::arg("out"), py::arg("scale"), py::arg("H"), py::arg("window"), py::arg("pool"),
         py::arg("sink"), py::arg("v_freq"), py::arg("vt") = py::none());
+  m.def("linear_attn_scratch", [](int64_t T, int64_t S, int64_t H, int64_t D, int64_t V) {
+    return (int64_t)vgate::linear_attn_scratch_floats((int)T, (int)S, (int)H, (int)D, (int)V);
+  }, "fp32 elements of scratch a linear_attn call over T rows and S sequences needs");
   m.def("linear_attn", &linear_attn, "decayed linear attention recurrence over state slots + norm + gate");
   m.def("moe_route", &moe_route, "sigmoid router: corrected top-k choice, normalised uncorrected weights");
   m.def("moe_sort", &moe_sort, "counting sort of (token, choice) pairs by expert");

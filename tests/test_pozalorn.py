@@ -608,3 +608,69 @@ def test_gelu_pair_gemm(device, f32):
     seq.gemm(a.to(d), w1.to(d), out, w2=w2.to(d), act=seq.ACT_GELU_TANH_MUL)
     want = oracle.gelu_tanh(a.float() @ w1.float().t()) * (a.float() @ w2.float().t())
     assert rel(out, want) < (1e-5 if f32 else 1e-2)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("act", ["silu", "gelu_tanh"])
+def test_glu_rows(device, act):
+    from vgate.ops import seq
+    g = torch.Generator().manual_seed(17)
+    d = torch.device(device)
+    gu = (torch.randn(7, 48, generator=g) * 2).to(torch.bfloat16)
+    out = torch.zeros(5, 24, dtype=torch.bfloat16, device=d)
+    seq.glu_rows(gu.to(d), out, seq.ACT_GELU_TANH_MUL if act == "gelu_tanh" else seq.ACT_SILU_MUL)
+    a, u = gu[:5, :24].float(), gu[:5, 24:].float()
+    want = (oracle.gelu_tanh(a) if act == "gelu_tanh" else oracle.silu(a)) * u
+    assert rel(out, want) < 5e-3
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("D,V", [(16, 24), (72, 40)])
+def test_linear_attention_long_portions(device, D, V):
+    """Portions of hundreds of tokens (on the GPU scanned in parallel chunks with a carry between them): a
+    lone sequence from position 0, its continuation from the slot's state, and two unequal sequences in one
+    step, all against the token-by-token recurrence. Decays down to ~0.01 per token: a chunk's decay product
+    underflows towards zero, which must stay harmless."""
+    from vgate.ops import seq
+    g = torch.Generator().manual_seed(18)
+    H = 2
+    d = torch.device(device)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=d)  # noqa: E731
+
+    def make(n):
+        q, k = (torch.randn(n, H * D, generator=g) * 0.5 for _ in range(2))
+        v, gt = (torch.randn(n, H * V, generator=g) for _ in range(2))
+        z = torch.randn(n, H * D, generator=g) * 3.0
+        return q, k, v, gt, z
+
+    nw = torch.randn(V, generator=g)
+    tau = 1.5
+
+    def want(x):
+        q, k, v, gt, z = x
+        n = q.shape[0]
+        a = (torch.sigmoid(z) ** (1.0 / tau)).view(n, H, D)
+        o = torch.stack([oracle.recurrence(q.view(n, H, D)[:, h], k.view(n, H, D)[:, h], v.view(n, H, V)[:, h], a[:, h])[0]
+                         for h in range(H)], 1)
+        return (oracle.rms_unit(o, 1e-5) * nw).reshape(n, -1) * oracle.silu(gt)
+
+    def step(parts, slots, ctx, state):
+        """parts: per sequence (tensors, first row, rows)."""
+        cat = lambda j: torch.cat([x[j][a: a + n] for x, a, n in parts]).to(d)  # noqa: E731
+        T = sum(n for _, _, n in parts)
+        out = torch.zeros(T, H * V, device=d)
+        qs = [0]
+        for _, _, n in parts:
+            qs.append(qs[-1] + n)
+        seq.linear_attn(cat(0), cat(1), cat(2), cat(3), cat(4), None, tau, 1.0, False, nw.to(d), False, True, state,
+                        i32(slots), i32(ctx), i32(qs), out, 1e-5)
+        return out.cpu()
+
+    A, B = make(700), make(90)
+    wa, wb = want(A), want(B)
+    state = torch.full((3, H, D, V), 3.0, device=d)
+    o1 = step([(A, 0, 450)], [2], [450], state)                       # lone sequence, chunked on the GPU
+    o2 = step([(A, 450, 200), (B, 0, 90)], [2, 0], [650, 90], state)  # continuation beside a new sequence
+    o3 = step([(A, 650, 50)], [2], [700], state)                      # short step: one pass from the slot
+    assert rel(torch.cat([o1, o2[:200], o3]), wa) < 5e-5
+    assert rel(o2[200:], wb) < 5e-5

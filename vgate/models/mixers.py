@@ -48,12 +48,14 @@ class Proj:
         self.pair_act = pair_act
         dev = torch.device(device)
         n_ok = (N // 2) % 64 == 0 if silu_pair else N % 64 == 0
-        # the packed kernels' pair epilogue is SiLU; another pair activation runs on the row-major GEMM
         self.packed = (USE_PACKED and allow_packed and not f32 and dev.type == "cuda" and n_ok and K % 64 == 0
-                       and K >= PACKED_MIN_K and (not silu_pair or pair_act == seq.ACT_SILU_MUL))
+                       and K >= PACKED_MIN_K)
+        # the packed kernels' pair epilogue is SiLU: another pair activation runs the stacked [gate; up]
+        # matrix as a plain packed GEMM and applies act(gate) * up in a row kernel
+        self.split_act = self.packed and silu_pair and pair_act != seq.ACT_SILU_MUL
         self.bias = None
         if self.packed:
-            self.lin = ops.Linear(w.to(dev, torch.bfloat16), kind="silu" if silu_pair else "plain",
+            self.lin = ops.Linear(w.to(dev, torch.bfloat16), kind="silu" if silu_pair and not self.split_act else "plain",
                                   bias=None if bias is None else bias.to(dev, torch.bfloat16).contiguous())
             self.w = None
         else:
@@ -67,6 +69,10 @@ class Proj:
 
     def __call__(self, x: torch.Tensor, out_f32: bool = False, act: int = 0, out: torch.Tensor | None = None) -> torch.Tensor:
         M = x.shape[0]
+        if self.split_act:
+            if out is None:
+                out = torch.empty(M, self.out_features, dtype=torch.bfloat16, device=x.device)
+            return seq.glu_rows(ops.linear(x, self.lin), out, self.pair_act)
         if self.packed and act == 0:
             return ops.linear(x, self.lin, out=out, out_f32=out_f32)
         dt = torch.float32 if (out_f32 or self.f32) else torch.bfloat16

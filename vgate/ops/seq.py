@@ -314,6 +314,16 @@ def cast_rows(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def glu_rows(gu: torch.Tensor, out: torch.Tensor, act: int) -> torch.Tensor:
+    """out = act(gu[:, :n]) * gu[:, n:] for a stacked [gate; up] projection (act: ACT_SILU_MUL or ACT_GELU_TANH_MUL)."""
+    if gu.is_cuda:
+        _C().glu_rows(gu, out, act)
+        return out
+    n = out.shape[1]
+    out.copy_(_act(gu[: out.shape[0], :n].float(), gu[: out.shape[0], n:].float(), act, 0.0, 0.0))
+    return out
+
+
 def post_norm_add(x, y1, w, eps: float, out, s1: float = 1.0, y2=None, s2: float = 1.0, act_out=None, hist=None,
                   planes: int = 0, coef=None, mix=None) -> None:
     """out = x + u / sqrt(mean(u^2) + eps) * w with u = s1 y1 [+ s2 y2], all in fp32 (out may be x).
@@ -460,7 +470,8 @@ def linear_attn(q, k, v, g, z, head_decay, tau: float, q_scale: float, in_silu: 
     position 0 starts from a zero state."""
     if q.is_cuda:
         H, D, V = state.shape[1], state.shape[2], state.shape[3]
-        scratch = torch.empty(q.shape[0] * H * (4 * D + 2 * V), dtype=torch.float32, device=q.device)
+        n = _C().linear_attn_scratch(q.shape[0], state_slots.numel(), H, D, V)
+        scratch = torch.empty(n, dtype=torch.float32, device=q.device)
         _C().linear_attn(q, k, v, g, z, head_decay, tau, q_scale, in_silu, nw, norm_all, gate_silu, state, state_slots,
                          context_lens, query_start, out, eps, scratch)
         return
