@@ -6,9 +6,10 @@
 // gate silu(g) or sigmoid(g). Key and value sizes may differ. Three launches:
 //   prep   (token, head) parallel: the fp32 per-channel triples {a, k, q_scale q} and the values.
 //   scan   the recurrence. Column v of S depends on no other column, so a head's value columns are split
-//          into slices of 8 and every (sequence, head, slice) is one wave: lane = (key group of eight,
-//          column), ceil(D / 8) state entries in registers; per token one FMA pair per entry and three
-//          lane exchanges for o. Tokens are staged through LDS, the next batch loaded into registers
+//          into slices of 8 NC and every (sequence, head, slice) is one wave: lane = (key group of eight,
+//          columns c + 8 n for n < NC), ceil(D / 8) x NC state entries in registers; per token one FMA pair
+//          per entry and three lane exchanges per column for o; one LDS read of a key channel's {a, k, q}
+//          serves the lane's NC columns (NC = 4 when there are enough waves without the finer split, else 1). Tokens are staged through LDS, the next batch loaded into registers
 //          while the current one computes. A sequence's tokens of the step run in order from the slot's
 //          state; a portion that starts at position 0 starts from zero, so a reused slot needs no clearing.
 //   finish token parallel: norm, norm weight, output gate, store in the activation dtype.
@@ -74,15 +75,17 @@ __device__ __forceinline__ bool locate_chunk(const LinearAttnArgs& p, int CH, in
   return false;
 }
 
-template <int DQ, int TC, int MODE>
+template <int DQ, int TC, int NC, int MODE>
 __global__ __launch_bounds__(64) void linear_scan_kernel(LinearAttnArgs p, const float4* __restrict__ vec,
                                                           const float* __restrict__ vals, float* __restrict__ oraw,
                                                           int CH, float* __restrict__ cstate, float* __restrict__ cdecay) {
-  constexpr int QV = DQ + 1;             // padded group stride: the groups' broadcast reads hit different banks
+  constexpr int QV = DQ + 1;              // padded group stride: the groups' broadcast reads hit different banks
   constexpr int NE = (8 * DQ + 63) / 64;  // channels a lane stages per token
+  constexpr int CW = 8 * NC;              // value columns of a wave: lane column + 8 n, n < NC
+  constexpr int NVL = (TC * CW + 63) / 64;
   __shared__ float4 lv[2][TC][8 * QV];
-  __shared__ float lvv[2][TC][8];
-  const int h = blockIdx.y, c0 = blockIdx.z * 8;
+  __shared__ float lvv[2][TC][CW];
+  const int h = blockIdx.y, c0 = blockIdx.z * CW;
   int s = blockIdx.x, t0, t1;
   if (MODE == SCAN_WHOLE) {
     t0 = p.query_start[s]; t1 = p.query_start[s + 1];
@@ -91,23 +94,26 @@ __global__ __launch_bounds__(64) void linear_scan_kernel(LinearAttnArgs p, const
     return;
   }
   const int D = p.D, V = p.V, lane = threadIdx.x;
-  const int q = lane >> 3, c = c0 + (lane & 7);
+  const int q = lane >> 3, cl = lane & 7;
   const int dq = (D + 7) >> 3;
   const int k0 = q * dq;
-  const bool con = c < V;
   // where this block's state starts from and goes to
   float* sp = MODE == SCAN_WHOLE ? p.state + ((int64_t)p.state_slots[s] * p.H + h) * D * V
                                  : cstate + ((int64_t)blockIdx.x * p.H + h) * D * V;
   const bool from_zero = MODE == SCAN_LOCAL ||
                          (MODE == SCAN_WHOLE && p.context_lens[s] - (t1 - t0) <= 0);
-  float S[DQ], A[MODE == SCAN_LOCAL ? DQ : 1];
+  float S[DQ][NC], A[MODE == SCAN_LOCAL ? DQ : 1];
 #pragma unroll
   for (int j = 0; j < DQ; ++j) {
-    S[j] = (con && j < dq && k0 + j < D && !from_zero) ? sp[(int64_t)(k0 + j) * V + c] : 0.f;
+#pragma unroll
+    for (int n = 0; n < NC; ++n) {
+      const int c = c0 + cl + 8 * n;
+      S[j][n] = (c < V && j < dq && k0 + j < D && !from_zero) ? sp[(int64_t)(k0 + j) * V + c] : 0.f;
+    }
     if (MODE == SCAN_LOCAL) A[j] = 1.f;
   }
   float4 pv[TC][NE];
-  float pvv[(TC * 8 + 63) / 64];
+  float pvv[NVL];
   auto fetch = [&](int tb) {
 #pragma unroll
     for (int i = 0; i < TC; ++i)
@@ -117,9 +123,11 @@ __global__ __launch_bounds__(64) void linear_scan_kernel(LinearAttnArgs p, const
         const bool ok = d < D && t < t1;
         pv[i][e] = ok ? vec[((int64_t)t * p.H + h) * D + d] : make_float4(0.f, 0.f, 0.f, 0.f);
       }
-    {  // TC x 8 values, lane -> (token, column)
-      const int t = tb + (lane >> 3), cc = c0 + (lane & 7);
-      pvv[0] = ((lane >> 3) < TC && t < t1 && cc < V) ? vals[((int64_t)t * p.H + h) * V + cc] : 0.f;
+#pragma unroll
+    for (int r = 0; r < NVL; ++r) {  // TC x CW values, lane -> (token, column)
+      const int e = lane + 64 * r;
+      const int t = tb + e / CW, cc = c0 + e % CW;
+      pvv[r] = (e < TC * CW && t < t1 && cc < V) ? vals[((int64_t)t * p.H + h) * V + cc] : 0.f;
     }
   };
   auto put = [&](int buf) {
@@ -130,7 +138,11 @@ __global__ __launch_bounds__(64) void linear_scan_kernel(LinearAttnArgs p, const
         const int d = lane + 64 * e;
         if (d < D) lv[buf][i][(d / dq) * QV + (d % dq)] = pv[i][e];
       }
-    if ((lane >> 3) < TC) lvv[buf][lane >> 3][lane & 7] = pvv[0];
+#pragma unroll
+    for (int r = 0; r < NVL; ++r) {
+      const int e = lane + 64 * r;
+      if (e < TC * CW) lvv[buf][e / CW][e % CW] = pvv[r];
+    }
   };
   // entries of channels past D are zeroed once and never written: the token loops run DQ iterations with
   // no bounds test (a = k = q = 0 leaves S and o alone)
@@ -148,20 +160,29 @@ __global__ __launch_bounds__(64) void linear_scan_kernel(LinearAttnArgs p, const
     for (int i = 0; i < TC; ++i) {
       if (i >= nt) break;
       const float4* tv = &lv[buf][i][q * QV];
-      const float vv = lvv[buf][i][lane & 7];
-      float o = 0.f;
+      float vv[NC], o[NC];
+#pragma unroll
+      for (int n = 0; n < NC; ++n) { vv[n] = lvv[buf][i][cl + 8 * n]; o[n] = 0.f; }
 #pragma unroll
       for (int j = 0; j < DQ; ++j) {
-        const float4 x = tv[j];  // {a, k, q}
-        S[j] = fmaf(x.y, vv, x.x * S[j]);
+        const float4 x = tv[j];  // {a, k, q}: one LDS read serves the lane's NC columns
+#pragma unroll
+        for (int n = 0; n < NC; ++n) {
+          S[j][n] = fmaf(x.y, vv[n], x.x * S[j][n]);
+          if (MODE != SCAN_LOCAL) o[n] = fmaf(x.z, S[j][n], o[n]);
+        }
         if (MODE == SCAN_LOCAL) A[j] *= x.x;
-        else o = fmaf(x.z, S[j], o);
       }
       if (MODE != SCAN_LOCAL) {
-        o += xor8(o);
-        o += xor16(o);
-        o += xor32(o);
-        if (con && q == 0) oraw[((int64_t)(tb + i) * p.H + h) * V + c] = o;
+#pragma unroll
+        for (int n = 0; n < NC; ++n) {
+          float r = o[n];
+          r += xor8(r);
+          r += xor16(r);
+          r += xor32(r);
+          const int c = c0 + cl + 8 * n;
+          if (c < V && q == 0) oraw[((int64_t)(tb + i) * p.H + h) * V + c] = r;
+        }
       }
     }
     if (more) {
@@ -173,16 +194,20 @@ __global__ __launch_bounds__(64) void linear_scan_kernel(LinearAttnArgs p, const
   if (MODE == SCAN_OUTPUT) return;
 #pragma unroll
   for (int j = 0; j < DQ; ++j)
-    if (con && j < dq && k0 + j < D) sp[(int64_t)(k0 + j) * V + c] = S[j];
-  if (MODE == SCAN_LOCAL && blockIdx.z == 0 && (lane & 7) == 0) {
+#pragma unroll
+    for (int n = 0; n < NC; ++n) {
+      const int c = c0 + cl + 8 * n;
+      if (c < V && j < dq && k0 + j < D) sp[(int64_t)(k0 + j) * V + c] = S[j][n];
+    }
+  if (MODE == SCAN_LOCAL && blockIdx.z == 0 && cl == 0) {
 #pragma unroll
     for (int j = 0; j < DQ; ++j)
       if (j < dq && k0 + j < D) cdecay[((int64_t)blockIdx.x * p.H + h) * D + k0 + j] = A[MODE == SCAN_LOCAL ? j : 0];
   }
 }
 
-// one workgroup per (sequence, head): I_0 = slot state (zero at position 0), I_(c+1) = diag(A_c) I_c + L_c;
-// cstate[c] becomes I_c, the slot the state after the last chunk
+// one thread per (sequence, head, state entry): I_0 = slot state (zero at position 0),
+// I_(c+1) = diag(A_c) I_c + L_c; cstate[c] becomes I_c, the slot the state after the last chunk
 __global__ __launch_bounds__(256) void linear_carry_kernel(LinearAttnArgs p, int CH, float* __restrict__ cstate,
                                                             const float* __restrict__ cdecay) {
   const int s = blockIdx.x, h = blockIdx.y;
@@ -198,7 +223,7 @@ __global__ __launch_bounds__(256) void linear_carry_kernel(LinearAttnArgs p, int
   const int D = p.D, V = p.V;
   const bool from_zero = p.context_lens[s] - (t1 - t0) <= 0;
   float* sp = p.state + ((int64_t)slot * p.H + h) * D * V;
-  for (int e = threadIdx.x; e < D * V; e += blockDim.x) {
+  for (int e = blockIdx.z * blockDim.x + threadIdx.x; e < D * V; e += gridDim.z * blockDim.x) {
     const int k = e / V;
     float cur = from_zero ? 0.f : sp[e];
     for (int c = 0; c < nc; ++c) {
@@ -243,21 +268,22 @@ __global__ __launch_bounds__(256) void linear_finish_kernel(LinearAttnArgs p, co
   }
 }
 
-template <int DQ, int TC>
+template <int DQ, int TC, int NC>
 void launch_scan(const LinearAttnArgs& a, int T, const float4* vec, const float* vals, float* oraw, int CH, float* cstate,
                  float* cdecay, hipStream_t st) {
-  const int cols = (a.V + 7) / 8;
+  const int cols = (a.V + 8 * NC - 1) / (8 * NC);
   if (CH <= 0) {
-    hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, SCAN_WHOLE>), dim3(a.S, a.H, cols), dim3(64), 0, st, a, vec, vals, oraw,
-                       0, nullptr, nullptr);
+    hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, NC, SCAN_WHOLE>), dim3(a.S, a.H, cols), dim3(64), 0, st, a, vec, vals,
+                       oraw, 0, nullptr, nullptr);
     return;
   }
   const int chunks = linear_attn_chunks(T, a.S, CH);
-  hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, SCAN_LOCAL>), dim3(chunks, a.H, cols), dim3(64), 0, st, a, vec, vals, oraw,
-                     CH, cstate, cdecay);
-  hipLaunchKernelGGL(linear_carry_kernel, dim3(a.S, a.H), dim3(256), 0, st, a, CH, cstate, cdecay);
-  hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, SCAN_OUTPUT>), dim3(chunks, a.H, cols), dim3(64), 0, st, a, vec, vals, oraw,
-                     CH, cstate, cdecay);
+  hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, NC, SCAN_LOCAL>), dim3(chunks, a.H, cols), dim3(64), 0, st, a, vec, vals,
+                     oraw, CH, cstate, cdecay);
+  const int ez = min(64, (a.D * a.V + 255) / 256);
+  hipLaunchKernelGGL(linear_carry_kernel, dim3(a.S, a.H, ez), dim3(256), 0, st, a, CH, cstate, cdecay);
+  hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, NC, SCAN_OUTPUT>), dim3(chunks, a.H, cols), dim3(64), 0, st, a, vec, vals,
+                     oraw, CH, cstate, cdecay);
 }
 
 }  // namespace
@@ -284,10 +310,14 @@ void launch_linear_attn(const LinearAttnArgs& a, int T, float* scratch, hipStrea
   float* cstate = oraw + nv;
   float* cdecay = cstate + (size_t)linear_attn_chunks(T, a.S, CH) * a.H * a.D * a.V;
   hipLaunchKernelGGL(linear_prep_kernel, dim3(T), dim3(256), 0, st, a, vec, vals);
-  if (a.D <= 32) launch_scan<4, 8>(a, T, vec, vals, oraw, CH, cstate, cdecay, st);
-  else if (a.D <= 64) launch_scan<8, 8>(a, T, vec, vals, oraw, CH, cstate, cdecay, st);
-  else if (a.D <= 128) launch_scan<16, 8>(a, T, vec, vals, oraw, CH, cstate, cdecay, st);
-  else launch_scan<32, 4>(a, T, vec, vals, oraw, CH, cstate, cdecay, st);
+  // columns per lane: few columns -> more waves (a small batch of decoded tokens needs them to fill the chip);
+  // wide values -> every LDS read of a key channel's {a, k, q} serves four columns
+  const bool wide = a.cols_per_lane > 0 ? a.cols_per_lane > 1
+                                        : a.V >= 32 && (int64_t)a.S * a.H * ((a.V + 31) / 32) * (CH > 0 ? T / CH + 1 : 1) >= 512;
+  if (a.D <= 32) { if (wide) launch_scan<4, 8, 4>(a, T, vec, vals, oraw, CH, cstate, cdecay, st); else launch_scan<4, 8, 1>(a, T, vec, vals, oraw, CH, cstate, cdecay, st); }
+  else if (a.D <= 64) { if (wide) launch_scan<8, 8, 4>(a, T, vec, vals, oraw, CH, cstate, cdecay, st); else launch_scan<8, 8, 1>(a, T, vec, vals, oraw, CH, cstate, cdecay, st); }
+  else if (a.D <= 128) { if (wide) launch_scan<16, 4, 4>(a, T, vec, vals, oraw, CH, cstate, cdecay, st); else launch_scan<16, 4, 1>(a, T, vec, vals, oraw, CH, cstate, cdecay, st); }
+  else { if (wide) launch_scan<32, 4, 2>(a, T, vec, vals, oraw, CH, cstate, cdecay, st); else launch_scan<32, 4, 1>(a, T, vec, vals, oraw, CH, cstate, cdecay, st); }
   hipLaunchKernelGGL(linear_finish_kernel, dim3(T), dim3(256), 0, st, a, oraw);
 }
 

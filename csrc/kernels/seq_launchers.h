@@ -138,6 +138,7 @@ struct LinearAttnArgs {
   const int32_t* state_slots = nullptr; const int32_t* context_lens = nullptr; const int32_t* query_start = nullptr;
   void* out = nullptr; int64_t ldo = 0;
   int S = 0, H = 0, D = 0, V = 0, f32 = 0;
+  int cols_per_lane = 0;                        // value columns per lane of the scan: 0 = by the launch's size, 1, or > 1 (wide)
 };
 // tokens per chunk a step of T rows over S sequences is scanned in (0: every sequence in one pass), the
 // chunks such a step has at most, and the scratch floats it needs

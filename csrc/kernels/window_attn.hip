@@ -18,8 +18,8 @@
 //               starts the running max at its logit and the running sum at 1. With turned values the
 //               normalised output is turned back by the query's position before it is stored.
 // window_attn, bf16 caches with head sizes in multiples of 8 up to 256: MFMA kernel. Rows are (token,
-//               query head of one key/value head) pairs of one sequence, 16 per wave, 4 independent waves
-//               per workgroup; keys in tiles of 32: first the pooled rows (two groups of 16, each lane
+//               query head of one key/value head) pairs of one sequence, 16 per workgroup, whose four
+//               waves take every fourth key tile and merge through LDS; keys in tiles of 32: first the pooled rows (two groups of 16, each lane
 //               addressing its own pooled row), then token tiles aligned to two whole pages.
 //                 S = Q K^T   v_mfma 16x16x32, Q fragments stationary, K fragments 16 B of a cached row
 //                 online softmax in fp32 (exp2 of log2(e)-scaled scores, per-lane partial row sums)
@@ -30,8 +30,6 @@
 //                             tiles the eight values are gathered from the pooled rows.
 //               Window, causal and pooled-block visibility are per-row masks on whole tiles, and tiles sit
 //               at fixed absolute key positions, so a row's sums do not depend on which rows share its wave.
-//               A sequence whose rows fit one wave (a decoded token) shares its tiles out over the
-//               workgroup's four waves, merged through LDS.
 // Every row of every kernel depends only on its own sequence's cache rows, in an order fixed by the
 // position, so results do not depend on how a prompt is cut or what else is in the batch.
 #include "common.h"
@@ -341,8 +339,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WindowArgs a, con
   __shared__ float mrg_o[16][16 * NCT];  // split mode: the merged weighted values of the 16 rows
   const int D = a.D, V = a.V, G = a.G, H = a.H, rep = H / G, g = blockIdx.y, P = a.pool;
   int s = -1, tile = 0, base = 0;
-  for (int i = 0; i < a.S; ++i) {  // (sequence, 64-row tile) of this workgroup
-    const int nt = ((a.query_start[i + 1] - a.query_start[i]) * rep + 63) / 64;
+  for (int i = 0; i < a.S; ++i) {  // (sequence, 16-row tile) of this workgroup
+    const int nt = ((a.query_start[i + 1] - a.query_start[i]) * rep + 15) / 16;
     if ((int)blockIdx.x < base + nt) { s = i; tile = blockIdx.x - base; break; }
     base += nt;
   }
@@ -351,9 +349,11 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WindowArgs a, con
   const int t0 = a.query_start[s], ntok = a.query_start[s + 1] - t0;
   const int pos0 = a.context_lens[s] - ntok;
   const int nrows = ntok * rep;
-  const bool split = nrows <= 16;  // workgroup-uniform: one row tile, key tiles shared out over the four waves
-  const int row0 = split ? 0 : tile * 64 + wv * 16;
-  if (row0 >= nrows) return;
+  // a workgroup owns 16 rows; its four waves take every fourth key tile of them and merge their partial
+  // (max, sum, weighted values) through LDS: four times the waves to hide the cache's latency behind
+  constexpr bool split = true;
+  const int row0 = tile * 16;
+  if (row0 >= nrows) return;  // (workgroup-uniform)
   const bf16_t* kc = reinterpret_cast<const bf16_t*>(a.kc);
   const bf16_t* kp = reinterpret_cast<const bf16_t*>(a.kp);
   const bf16_t* vp = reinterpret_cast<const bf16_t*>(a.vp);
@@ -560,7 +560,7 @@ template <int NCT, int NQF>
 void launch_window_mfma(const WindowArgs& a, const void* q, float scale, const void* vt, int num_pages, void* out,
                         hipStream_t st) {
   const int rep = a.H / a.G;
-  const int blocks = (a.T * rep + 63) / 64 + a.S;
+  const int blocks = (a.T * rep + 15) / 16 + a.S;
   hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF>), dim3(blocks, a.G), dim3(256), 0, st, a,
                      reinterpret_cast<const bf16_t*>(q), scale * 1.4426950408889634f, reinterpret_cast<const bf16_t*>(vt),
                      num_pages, reinterpret_cast<bf16_t*>(out));

@@ -417,8 +417,10 @@ void window_attn(const Tensor& q, const Tensor& kc, const Tensor& vc, const OptT
 void linear_attn(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& g, const OptT& z, const OptT& head_decay,
                  double tau, double q_scale, bool in_silu, const Tensor& nw, bool norm_all, bool gate_silu, Tensor& state,
                  const Tensor& state_slots, const Tensor& context_lens, const Tensor& query_start, Tensor& out, double eps,
-                 Tensor& scratch) {
+                 Tensor& scratch, int64_t cols_per_lane) {
   vgate::LinearAttnArgs p;
+  TORCH_CHECK(cols_per_lane >= 0 && cols_per_lane <= 4, "linear_attn: cols_per_lane 0 (auto), 1 or 4");
+  p.cols_per_lane = (int)cols_per_lane;
   p.f32 = act_f32(q, "q");
   TORCH_CHECK(state.is_cuda() && state.scalar_type() == torch::kFloat32 && state.is_contiguous() && state.dim() == 4,
               "linear_attn: state fp32 [slots, H, D, V]");
@@ -535,7 +537,11 @@ void bind_seq(pybind11::module& m) {
   m.def("linear_attn_scratch", [](int64_t T, int64_t S, int64_t H, int64_t D, int64_t V) {
     return (int64_t)vgate::linear_attn_scratch_floats((int)T, (int)S, (int)H, (int)D, (int)V);
   }, "fp32 elements of scratch a linear_attn call over T rows and S sequences needs");
-  m.def("linear_attn", &linear_attn, "decayed linear attention recurrence over state slots + norm + gate");
+  m.def("linear_attn", &linear_attn, "decayed linear attention recurrence over state slots + norm + gate", py::arg("q"),
+        py::arg("k"), py::arg("v"), py::arg("g"), py::arg("z"), py::arg("head_decay"), py::arg("tau"), py::arg("q_scale"),
+        py::arg("in_silu"), py::arg("nw"), py::arg("norm_all"), py::arg("gate_silu"), py::arg("state"), py::arg("state_slots"),
+        py::arg("context_lens"), py::arg("query_start"), py::arg("out"), py::arg("eps"), py::arg("scratch"),
+        py::arg("cols_per_lane") = 0);
   m.def("moe_route", &moe_route, "sigmoid router: corrected top-k choice, normalised uncorrected weights");
   m.def("moe_sort", &moe_sort, "counting sort of (token, choice) pairs by expert");
   m.def("moe_combine", &moe_combine, "weighted sum of a token's expert rows");

@@ -555,7 +555,7 @@ def test_linear_attention_state_carry_and_slots(device, D, V, channel):
         o = (oracle.rms_unit(o.reshape(n, -1), 1e-5) * nw) if norm_all else (oracle.rms_unit(o, 1e-5) * nw).reshape(n, -1)
         want = o * (oracle.silu(gt) if gate_silu else torch.sigmoid(gt))
 
-        def run(cuts, slot, state, extra=None):
+        def run(cuts, slot, state, cols=0):
             out = torch.zeros(n, H * V, device=d)
             at = 0
             for c in cuts:
@@ -563,14 +563,15 @@ def test_linear_attention_state_carry_and_slots(device, D, V, channel):
                 sl = slice(at, at + c)
                 seq.linear_attn(q[sl].to(d), k[sl].to(d), v[sl].to(d), gt[sl].to(d), z[sl].to(d) if channel else None,
                                 None if channel else decay.to(d), tau, qs_, in_silu, nw.to(d), norm_all, gate_silu, state,
-                                i32([slot]), i32([at + c]), i32([0, c]), out[sl], 1e-5)
+                                i32([slot]), i32([at + c]), i32([0, c]), out[sl], 1e-5, cols_per_lane=cols)
                 at += c
             return out.cpu()
 
         state = torch.full((3, H, D, V), 5.0, device=d)   # garbage a previous owner left
         assert rel(run([n], 1, state), want) < 3e-5
         assert rel(run([3, 1, 1, 9, 2, 13], 2, state), want) < 3e-5
-        assert bool((state[0] == 5.0).all())
+        assert rel(run([3, 1, 1, 9, 2, 13], 0, state, cols=4), want) < 3e-5
+        assert bool((state[0, 0, 0, :] != 5.0).all())
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -654,7 +655,7 @@ def test_linear_attention_long_portions(device, D, V):
                          for h in range(H)], 1)
         return (oracle.rms_unit(o, 1e-5) * nw).reshape(n, -1) * oracle.silu(gt)
 
-    def step(parts, slots, ctx, state):
+    def step(parts, slots, ctx, state, cols=0):
         """parts: per sequence (tensors, first row, rows)."""
         cat = lambda j: torch.cat([x[j][a: a + n] for x, a, n in parts]).to(d)  # noqa: E731
         T = sum(n for _, _, n in parts)
@@ -663,14 +664,15 @@ def test_linear_attention_long_portions(device, D, V):
         for _, _, n in parts:
             qs.append(qs[-1] + n)
         seq.linear_attn(cat(0), cat(1), cat(2), cat(3), cat(4), None, tau, 1.0, False, nw.to(d), False, True, state,
-                        i32(slots), i32(ctx), i32(qs), out, 1e-5)
+                        i32(slots), i32(ctx), i32(qs), out, 1e-5, cols_per_lane=cols)
         return out.cpu()
 
     A, B = make(700), make(90)
     wa, wb = want(A), want(B)
-    state = torch.full((3, H, D, V), 3.0, device=d)
-    o1 = step([(A, 0, 450)], [2], [450], state)                       # lone sequence, chunked on the GPU
-    o2 = step([(A, 450, 200), (B, 0, 90)], [2, 0], [650, 90], state)  # continuation beside a new sequence
-    o3 = step([(A, 650, 50)], [2], [700], state)                      # short step: one pass from the slot
-    assert rel(torch.cat([o1, o2[:200], o3]), wa) < 5e-5
-    assert rel(o2[200:], wb) < 5e-5
+    for cols in (0, 1, 4):   # columns a lane of the GPU scan keeps (0: by the launch's size)
+        state = torch.full((3, H, D, V), 3.0, device=d)
+        o1 = step([(A, 0, 450)], [2], [450], state, cols)                       # lone sequence, chunked on the GPU
+        o2 = step([(A, 450, 200), (B, 0, 90)], [2, 0], [650, 90], state, cols)  # continuation beside a new sequence
+        o3 = step([(A, 650, 50)], [2], [700], state, cols)                      # short step: one pass from the slot
+        assert rel(torch.cat([o1, o2[:200], o3]), wa) < 5e-5, cols
+        assert rel(o2[200:], wb) < 5e-5, cols

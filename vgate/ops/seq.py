@@ -461,19 +461,20 @@ def window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out,
 # ---------------------------------------------------------------------------------- linear attention
 def linear_attn(q, k, v, g, z, head_decay, tau: float, q_scale: float, in_silu: bool, nw, norm_all: bool,
                 gate_silu: bool, state, state_slots, context_lens, query_start, out, eps: float,
-                num_seqs: int | None = None) -> None:
+                num_seqs: int | None = None, cols_per_lane: int = 0) -> None:
     """Decayed outer-product recurrence over state slots, state [slots, H, D, V] fp32:
         S <- diag(a_t) S + k_t v_t^T,  o_t = S^T (q_scale q_t)
     a_t = sigmoid(z_t)^(1 / tau) per key channel (``z`` fp32 [T, H * D]) or the constant head_decay[h];
     ``in_silu``: silu on q, k, v. Then RMS norm of o (per head with a [V] weight, or with ``norm_all`` over
     the concatenated heads with a [H * V] weight), times silu(g) or sigmoid(g). A portion that starts at
-    position 0 starts from a zero state."""
+    position 0 starts from a zero state. ``cols_per_lane`` (GPU): value columns a lane of the scan keeps, 0 =
+    chosen by the launch's size."""
     if q.is_cuda:
         H, D, V = state.shape[1], state.shape[2], state.shape[3]
         n = _C().linear_attn_scratch(q.shape[0], state_slots.numel(), H, D, V)
         scratch = torch.empty(n, dtype=torch.float32, device=q.device)
         _C().linear_attn(q, k, v, g, z, head_decay, tau, q_scale, in_silu, nw, norm_all, gate_silu, state, state_slots,
-                         context_lens, query_start, out, eps, scratch)
+                         context_lens, query_start, out, eps, scratch, cols_per_lane)
         return
     H, D, V = state.shape[1], state.shape[2], state.shape[3]
     S = state_slots.numel() if num_seqs is None else num_seqs
