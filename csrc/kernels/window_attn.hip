@@ -330,12 +330,13 @@ __device__ __forceinline__ float group16_sum(float v) {
 // end or the value's last column is read from a clamped address: its partner (zero Q fragment) or its
 // output column (never stored) makes the value irrelevant, and cached values are always finite.
 constexpr int LG = 4;
-template <int NCT, int NQF>
-__global__ __launch_bounds__(256) void window_attn_mfma_kernel(WindowArgs a, const bf16_t* __restrict__ q,
+// NW: waves of a workgroup, which share out the key tiles of its 16 rows
+template <int NCT, int NQF, int NW>
+__global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a, const bf16_t* __restrict__ q,
                                                                 float scale_log2e, const bf16_t* __restrict__ vt,
                                                                 int num_pages, bf16_t* __restrict__ out) {
-  __shared__ __attribute__((aligned(16))) bf16_t pl[4][16][40];
-  __shared__ float mrg_m[4][16], mrg_l[4][16];
+  __shared__ __attribute__((aligned(16))) bf16_t pl[NW][16][40];
+  __shared__ float mrg_m[NW][16], mrg_l[NW][16];
   __shared__ float mrg_o[16][16 * NCT];  // split mode: the merged weighted values of the 16 rows
   const int D = a.D, V = a.V, G = a.G, H = a.H, rep = H / G, g = blockIdx.y, P = a.pool;
   int s = -1, tile = 0, base = 0;
@@ -391,7 +392,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WindowArgs a, con
 #pragma unroll
   for (int ct = 0; ct < NCT; ++ct) O[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int32_t* bt = a.block_tables + (int64_t)s * a.max_blocks;
-  for (int ti = split ? wv : 0; ti < ntiles; ti += split ? 4 : 1) {
+  for (int ti = split ? wv : 0; ti < ntiles; ti += split ? NW : 1) {
     const bool pooled = ti < ntp;  // wave-uniform
     int kbase, pg0 = 0, pg1 = 0;
     const bf16_t* k0p;
@@ -502,16 +503,16 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WindowArgs a, con
       const int r = 4 * lg + i;
       float M = mrg_m[0][r];
 #pragma unroll
-      for (int w = 1; w < 4; ++w) M = fmaxf(M, mrg_m[w][r]);
+      for (int w = 1; w < NW; ++w) M = fmaxf(M, mrg_m[w][r]);
       const float Ms = (M == -INFINITY) ? 0.f : M;  // (rows past the sequence's last)
       float L = 0.f;
 #pragma unroll
-      for (int w = 0; w < 4; ++w) L += mrg_l[w][r] * exp2f(mrg_m[w][r] - Ms);  // a wave that saw no key: l = 0, exp2(-inf) = 0
+      for (int w = 0; w < NW; ++w) L += mrg_l[w][r] * exp2f(mrg_m[w][r] - Ms);  // a wave that saw no key: l = 0, exp2(-inf) = 0
       f[i] = exp2f(m[i] - Ms);
       lsum[i] = L;                // the merged row sum (the same in every lane of the row)
       m[i] = M;
     }
-    for (int w = 0; w < 4; ++w) {  // waves add their scaled partials in turn
+    for (int w = 0; w < NW; ++w) {  // waves add their scaled partials in turn
       if (wv == w) {
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct)
@@ -561,9 +562,15 @@ void launch_window_mfma(const WindowArgs& a, const void* q, float scale, const v
                         hipStream_t st) {
   const int rep = a.H / a.G;
   const int blocks = (a.T * rep + 15) / 16 + a.S;
-  hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF>), dim3(blocks, a.G), dim3(256), 0, st, a,
-                     reinterpret_cast<const bf16_t*>(q), scale * 1.4426950408889634f, reinterpret_cast<const bf16_t*>(vt),
-                     num_pages, reinterpret_cast<bf16_t*>(out));
+  const bf16_t* qp = reinterpret_cast<const bf16_t*>(q);
+  const bf16_t* vp = reinterpret_cast<const bf16_t*>(vt);
+  bf16_t* op = reinterpret_cast<bf16_t*>(out);
+  const float sl = scale * 1.4426950408889634f;
+  // few rows per sequence (decoded tokens): few workgroups, so eight waves each stream the keys; else four
+  if ((int64_t)a.T * rep <= 16 * (int64_t)a.S)
+    hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 8>), dim3(blocks, a.G), dim3(512), 0, st, a, qp, sl, vp, num_pages, op);
+  else
+    hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 4>), dim3(blocks, a.G), dim3(256), 0, st, a, qp, sl, vp, num_pages, op);
 }
 
 int heads_per_block(const WindowArgs& a) {
