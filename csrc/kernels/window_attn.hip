@@ -9,7 +9,7 @@
 //               fp32 statistics), interleaved-pair rotation of the leading rot_dims entries of every head
 //               (angle = position * inv_freq in fp32, full-range sin / cos), values optionally turned over
 //               all of V, the paged stores, and the prepared query rows.
-// window_pool   one workgroup per token whose position completes a block: fp32 mean of the block's P
+// window_pool   workgroups of 256 elements per token whose position completes a block: fp32 mean of the block's P
 //               cached rows, in position order, into the pooled row. It runs after window_write of the
 //               same step, so a block completed inside a prompt portion reads rows of that portion too.
 // window_attn   one workgroup per (token, key/value head, chunk of its query heads): the keys a query
@@ -132,7 +132,16 @@ __global__ __launch_bounds__(256) void window_write_kernel(WindowArgs a, const v
   }
 }
 
+template <typename T>
+__device__ __forceinline__ float ld_as_float(const T* p, int64_t i);
+template <>
+__device__ __forceinline__ float ld_as_float<float>(const float* p, int64_t i) { return p[i]; }
+template <>
+__device__ __forceinline__ float ld_as_float<bf16_t>(const bf16_t* p, int64_t i) { return bf2f(p[i]); }
+
+template <typename T>
 __global__ __launch_bounds__(256) void window_pool_kernel(WindowArgs a) {
+  __shared__ int32_t pages[64];  // the pages of the block's rows, a stretch of up to 64 at a time
   const int t = blockIdx.x;
   if (t >= a.query_start[a.S]) return;
   const int e = a.positions[t], P = a.pool;
@@ -142,16 +151,40 @@ __global__ __launch_bounds__(256) void window_pool_kernel(WindowArgs a) {
   const int G = a.G, D = a.D, V = a.V, page = a.page;
   const int64_t dpg = bt[e / page];
   const int drow = (e % page) / P;
-  for (int x = threadIdx.x; x < G * (D + V); x += blockDim.x) {
+  const int j0 = e + 1 - P, pg_first = j0 / page, npg = e / page - pg_first + 1;
+  const int nx = G * (D + V);
+  // every thread sums one element over the block's rows in position order; the page ids come from LDS, so a
+  // row's loads do not wait for a block-table load and sixteen rows are in flight (the rows were written by
+  // the launch before, mostly on other XCDs: each batch costs a trip past the L2)
+  {  // blockIdx.y: which 256 elements
+    const int x = blockIdx.y * blockDim.x + threadIdx.x;
+    const bool on = x < nx;
     const bool isk = x < G * D;
     const int y = isk ? x : x - G * D;
     const int w = isk ? D : V;
-    const int g = y / w, i = y % w;
-    const void* src = isk ? a.kc : a.vc;
+    const int g = on ? y / w : 0, i = on ? y % w : 0;
+    const T* src = reinterpret_cast<const T*>(isk ? a.kc : a.vc);
     float sum = 0.f;
-    for (int j = e + 1 - P; j <= e; ++j)
-      sum += ldx(src, (((int64_t)bt[j / page] * G + g) * page + j % page) * w + i, a.f32);
-    stx(isk ? a.kp : a.vp, ((dpg * G + g) * a.npool + drow) * w + i, a.f32, sum / (float)P);
+    for (int pb = 0; pb < npg; pb += 64) {
+      __syncthreads();
+      if ((int)threadIdx.x < min(64, npg - pb)) pages[threadIdx.x] = bt[pg_first + pb + threadIdx.x];
+      __syncthreads();
+      const int ja = max(j0, (pg_first + pb) * page), jb = min(e, (pg_first + min(npg, pb + 64)) * page - 1);
+      if (on) {
+        for (int j = ja; j <= jb; j += 16) {  // sixteen rows' loads in flight, added in position order
+          float v[16];
+#pragma unroll
+          for (int u = 0; u < 16; ++u) {
+            const int jj = min(j + u, jb);
+            v[u] = ld_as_float<T>(src, (((int64_t)pages[jj / page - pg_first - pb] * G + g) * page + jj % page) * w + i);
+          }
+#pragma unroll
+          for (int u = 0; u < 16; ++u)
+            if (j + u <= jb) sum += v[u];
+        }
+      }
+    }
+    if (on) stx(isk ? a.kp : a.vp, ((dpg * G + g) * a.npool + drow) * w + i, a.f32, sum / (float)P);
   }
 }
 
@@ -604,7 +637,9 @@ void launch_window_write(const WindowArgs& a, const void* q, int64_t ldq, const 
 
 void launch_window_pool(const WindowArgs& a, hipStream_t st) {
   if (a.T <= 0 || a.pool <= 0 || a.S <= 0) return;
-  hipLaunchKernelGGL(window_pool_kernel, dim3(a.T), dim3(256), 0, st, a);
+  const dim3 grid(a.T, (a.G * (a.D + a.V) + 255) / 256);
+  if (a.f32) hipLaunchKernelGGL(window_pool_kernel<float>, grid, dim3(256), 0, st, a);
+  else hipLaunchKernelGGL(window_pool_kernel<bf16_t>, grid, dim3(256), 0, st, a);
 }
 
 void launch_window_attn(const WindowArgs& a, const void* q, float scale, void* out, const void* vt, int num_pages,
