@@ -370,7 +370,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
                                                                 int num_pages, bf16_t* __restrict__ out) {
   __shared__ __attribute__((aligned(16))) bf16_t pl[NW][16][40];
   __shared__ float mrg_m[NW][16], mrg_l[NW][16];
-  __shared__ float mrg_o[16][16 * NCT];  // split mode: the merged weighted values of the 16 rows
+  __shared__ float mrg_o[16][16 * NCT];  // the merged weighted values of the 16 rows
   const int D = a.D, V = a.V, G = a.G, H = a.H, rep = H / G, g = blockIdx.y, P = a.pool;
   int s = -1, tile = 0, base = 0;
   for (int i = 0; i < a.S; ++i) {  // (sequence, 16-row tile) of this workgroup
@@ -385,7 +385,6 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
   const int nrows = ntok * rep;
   // a workgroup owns 16 rows; its four waves take every fourth key tile of them and merge their partial
   // (max, sum, weighted values) through LDS: four times the waves to hide the cache's latency behind
-  constexpr bool split = true;
   const int row0 = tile * 16;
   if (row0 >= nrows) return;  // (workgroup-uniform)
   const bf16_t* kc = reinterpret_cast<const bf16_t*>(a.kc);
@@ -411,7 +410,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
     hi[i] = ok ? p : -1;
     lo[i] = p - a.window + 1;
     nbv[i] = (ok && P > 0) ? max(0, lo[i]) / P : 0;
-    const bool sk = ok && a.sink != nullptr && (!split || wv == 0);  // the sink counts once
+    const bool sk = ok && a.sink != nullptr && wv == 0;  // the sink counts once
     m[i] = sk ? a.sink[g * rep + r % rep] * 1.4426950408889634f : -INFINITY;
     lsum[i] = (sk && lr == 0) ? 1.f : 0.f;
   }
@@ -425,7 +424,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
 #pragma unroll
   for (int ct = 0; ct < NCT; ++ct) O[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int32_t* bt = a.block_tables + (int64_t)s * a.max_blocks;
-  for (int ti = split ? wv : 0; ti < ntiles; ti += split ? NW : 1) {
+  for (int ti = wv; ti < ntiles; ti += NW) {
     const bool pooled = ti < ntp;  // wave-uniform
     int kbase, pg0 = 0, pg1 = 0;
     const bf16_t* k0p;
@@ -523,7 +522,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // P tile read before the next tile overwrites it
   }
-  if (split) {
+  {  // merge the waves' partials of every row
     float f[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -558,25 +557,25 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
       }
       __syncthreads();
     }
-    if (wv != 0) return;
-#pragma unroll
-    for (int ct = 0; ct < NCT; ++ct)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) O[ct][i] = mrg_o[4 * lg + i][16 * ct + lr];
   }
+  // eight waves (decoded tokens) share the epilogue out: wave w finishes the column tiles ct = w, w + NW, ..;
+  // with four (prompt portions) wave 0 finishes all of them: the shared form costs four registers there, which
+  // is the step from four waves per SIMD to three (measured 167 us against 109 us)
+  constexpr bool SHARE = NW > 4;
+  if (!SHARE && wv != 0) return;
   const int vrot = a.v_freq != nullptr ? 2 * (V / 2) : 0;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const float tot = split ? lsum[i] : group16_sum(lsum[i]);
-    const float inv = 1.f / tot;
+    const float inv = 1.f / lsum[i];
     const int r = row0 + 4 * lg + i;
     const bool ok = r < nrows;
     const float fp = -(float)(pos0 + (ok ? r / rep : 0));
     bf16_t* orow = out + ((int64_t)(t0 + (ok ? r / rep : 0)) * H + g * rep + (ok ? r % rep : 0)) * V;
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct) {
+      if (SHARE && ct % NW != wv) continue;  // wave-uniform
       const int col = 16 * ct + lr;
-      float y = O[ct][i] * inv;
+      float y = mrg_o[4 * lg + i][col] * inv;
       if (vrot > 0) {  // turn the pair (even column, the next one) back by the row's position: the partner is lane l ^ 1
         const float other = __shfl_xor(y, 1, 64);
         if (col < vrot) {
