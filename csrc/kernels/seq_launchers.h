@@ -101,6 +101,7 @@ struct WindowArgs {
   int page = 0, npool = 0;              // tokens per page; pooled rows per page (0: no pooled caches)
   int rot_dims = 0, window = 0, pool = 0;
   int f32 = 0, T = 0, S = 0, max_blocks = 0;
+  int prefill_kernel = 0;               // MFMA path, prompt portions: 0 LDS-staged tiles (64 rows), 1 split tiles (16 rows)
   const float* inv_freq = nullptr;      // [rot_dims / 2]
   const float* v_freq = nullptr;        // [V / 2]: values are turned by their position (null: not)
   const float* sink = nullptr;          // [H] logits that only enter the softmax denominator (null: none)

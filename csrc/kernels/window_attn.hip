@@ -589,6 +589,231 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
   }
 }
 
+// Prompt portions: 64 rows per workgroup (16 per wave). The waves walk the same key tiles; a token tile's keys
+// and transposed values are brought into LDS once per workgroup (two buffers: tile t + 1 is asked for before
+// tile t is computed, written after it, one barrier per tile), and every wave takes its fragments from there.
+// Pooled tiles come first and are read straight from the pooled caches by each wave, as in the kernel above.
+template <int NCT, int NQF>
+__global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, const bf16_t* __restrict__ q,
+                                                                 float scale_log2e, const bf16_t* __restrict__ vt,
+                                                                 int num_pages, bf16_t* __restrict__ out) {
+  constexpr int DP = 32 * NQF + 8;  // padded row of a staged key (bf16): rows 16 B apart in the banks
+  constexpr int VP = 40;            // padded row of a staged value column: 32 keys + 8
+  constexpr int NKC = (32 * 4 * NQF + 255) / 256, NVC = (4 * 16 * NCT + 255) / 256;  // 16-B pieces per thread
+  __shared__ __attribute__((aligned(16))) bf16_t kl[2][32][DP];
+  __shared__ __attribute__((aligned(16))) bf16_t vl[2][16 * NCT][VP];
+  __shared__ __attribute__((aligned(16))) bf16_t pl[4][16][40];
+  const int D = a.D, V = a.V, G = a.G, H = a.H, rep = H / G, g = blockIdx.y, P = a.pool;
+  int s = -1, tile = 0, base = 0;
+  for (int i = 0; i < a.S; ++i) {  // (sequence, 64-row tile) of this workgroup
+    const int nt = ((a.query_start[i + 1] - a.query_start[i]) * rep + 63) / 64;
+    if ((int)blockIdx.x < base + nt) { s = i; tile = blockIdx.x - base; break; }
+    base += nt;
+  }
+  if (s < 0) return;
+  const int tid = threadIdx.x, wv = tid >> 6, l = tid & 63, lr = l & 15, lg = l >> 4;
+  const int t0 = a.query_start[s], ntok = a.query_start[s + 1] - t0;
+  const int pos0 = a.context_lens[s] - ntok;
+  const int nrows = ntok * rep;
+  const int rowb = tile * 64;        // first row of the workgroup
+  if (rowb >= nrows) return;
+  const int row0 = rowb + wv * 16;   // first row of the wave
+  const bool active = row0 < nrows;  // wave-uniform; an idle wave still stages tiles and meets the barriers
+  const bf16_t* kc = reinterpret_cast<const bf16_t*>(a.kc);
+  const bf16_t* kp = reinterpret_cast<const bf16_t*>(a.kp);
+  const bf16_t* vp = reinterpret_cast<const bf16_t*>(a.vp);
+  const int nqf = (D + 31) >> 5, nct = (V + 15) >> 4, d8 = D >> 3;
+  for (int e = tid; e < 2 * 32 * DP / 8; e += 256) reinterpret_cast<uint4*>(&kl[0][0][0])[e] = make_uint4(0, 0, 0, 0);
+  for (int e = tid; e < 2 * 16 * NCT * VP / 8; e += 256) reinterpret_cast<uint4*>(&vl[0][0][0])[e] = make_uint4(0, 0, 0, 0);
+  bf16x8 qf[NQF];
+  {
+    const int r = row0 + lr;
+    const bool ok = r < nrows;
+    const bf16_t* qrow = q + ((int64_t)(t0 + (ok ? r / rep : 0)) * H + g * rep + (ok ? r % rep : 0)) * D;
+#pragma unroll
+    for (int kk = 0; kk < NQF; ++kk) qf[kk] = frag16(qrow, 32 * kk + 8 * lg, D, ok && kk < nqf);
+  }
+  int hi[4], lo[4], nbv[4];
+  float m[4], lsum[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = row0 + 4 * lg + i;
+    const bool ok = r < nrows;
+    const int p = pos0 + (ok ? r / rep : 0);
+    hi[i] = ok ? p : -1;
+    lo[i] = p - a.window + 1;
+    nbv[i] = (ok && P > 0) ? max(0, lo[i]) / P : 0;
+    const bool sk = ok && a.sink != nullptr;
+    m[i] = sk ? a.sink[g * rep + r % rep] * 1.4426950408889634f : -INFINITY;
+    lsum[i] = (sk && lr == 0) ? 1.f : 0.f;
+  }
+  // workgroup-uniform key ranges
+  const int lastb = min(rowb + 63, nrows - 1);
+  const int pminb = pos0 + rowb / rep, pmaxb = pos0 + lastb / rep;
+  const int jt0 = max(0, pminb - a.window + 1) >> 5, jt1 = pmaxb >> 5;
+  // wave-uniform: what this wave's rows can see at all
+  const int lastw = min(row0 + 15, nrows - 1);
+  const int pminw = pos0 + row0 / rep, pmaxw = pos0 + lastw / rep;
+  const int klow = max(0, pminw - a.window + 1);
+  const int nbmax = (active && P > 0) ? max(0, pmaxw - a.window + 1) / P : 0;
+  f32x4 O[NCT];
+#pragma unroll
+  for (int ct = 0; ct < NCT; ++ct) O[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int32_t* bt = a.block_tables + (int64_t)s * a.max_blocks;
+
+  // one tile's scores -> weights -> P in LDS; returns nothing, updates m, lsum, O scale
+  auto softmax_tile = [&](const f32x4& s0, const f32x4& s1, int kbase, bool pooled) {
+    float al[4];
+    const int c0 = kbase + lr, c1 = kbase + 16 + lr;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool vis0 = pooled ? c0 < nbv[i] : (c0 >= lo[i] && c0 <= hi[i]);
+      const bool vis1 = pooled ? c1 < nbv[i] : (c1 >= lo[i] && c1 <= hi[i]);
+      const float v0 = vis0 ? s0[i] * scale_log2e : -INFINITY;
+      const float v1 = vis1 ? s1[i] * scale_log2e : -INFINITY;
+      const float mnew = fmaxf(m[i], group16_max(fmaxf(v0, v1)));
+      const float ms = (mnew == -INFINITY) ? 0.f : mnew;
+      al[i] = exp2f(m[i] - ms);
+      const float p0 = exp2f(v0 - ms), p1 = exp2f(v1 - ms);
+      lsum[i] = lsum[i] * al[i] + p0 + p1;
+      m[i] = mnew;
+      pl[wv][4 * lg + i][lr] = f2bf(p0);
+      pl[wv][4 * lg + i][16 + lr] = f2bf(p1);
+    }
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) O[ct][i] *= al[i];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's P tile is written (LDS is in order per wave)
+  };
+
+  // pooled tiles: each wave for itself, straight from the pooled caches
+  for (int ti = 0; ti < ((nbmax + 31) >> 5); ++ti) {
+    const int kbase = 32 * ti;
+    const int e0 = min(kbase + lr, nbmax - 1) * P + P - 1, e1 = min(kbase + 16 + lr, nbmax - 1) * P + P - 1;
+    const int q0 = min(max(bt[e0 >> 4], 0), num_pages - 1), q1 = min(max(bt[e1 >> 4], 0), num_pages - 1);
+    const bf16_t* k0p = kp + (((int64_t)q0 * G + g) * a.npool + (e0 & 15) / P) * D;
+    const bf16_t* k1p = kp + (((int64_t)q1 * G + g) * a.npool + (e1 & 15) / P) * D;
+    f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kk = 0; kk < NQF; ++kk)
+      if (kk < nqf) {
+        const int off = min(32 * kk + 8 * lg, D - 8);
+        s0 = mfma16(qf[kk], as_bf16x8(ld16(k0p + off)), s0);
+        s1 = mfma16(qf[kk], as_bf16x8(ld16(k1p + off)), s1);
+      }
+    softmax_tile(s0, s1, kbase, true);
+    const bf16x8 pf = as_bf16x8(*reinterpret_cast<const uint4*>(&pl[wv][lr][8 * lg]));
+    int64_t ro[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int e1b = min(kbase + 8 * lg + e, nbmax - 1) * P + P - 1;
+      const int pq = min(max(bt[e1b >> 4], 0), num_pages - 1);
+      ro[e] = (((int64_t)pq * G + g) * a.npool + (e1b & 15) / P) * V;
+    }
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct)
+      if (ct < nct) {
+        const int col = min(16 * ct + lr, V - 1);
+        uint32_t w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w[j] = (uint32_t)vp[ro[2 * j] + col] | ((uint32_t)vp[ro[2 * j + 1] + col] << 16);
+        O[ct] = mfma16(pf, as_bf16x8(make_uint4(w[0], w[1], w[2], w[3])), O[ct]);
+      }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // P tile read before the next tile overwrites it
+  }
+
+  // token tiles through LDS (asking for tile t + 2 as well, through a second register set, was measured: 164
+  // registers, 139 us against 85 us)
+  uint4 kr[NKC], vr[NVC];
+  auto fetch = [&](int jt) {
+    const int kbase = 32 * jt;
+    int pg0 = bt[kbase >> 4];
+    int pg1 = (kbase + 16 <= pmaxb) ? bt[(kbase >> 4) + 1] : pg0;
+    pg0 = min(max(pg0, 0), num_pages - 1);
+    pg1 = min(max(pg1, 0), num_pages - 1);
+#pragma unroll
+    for (int u = 0; u < NKC; ++u) {
+      const int c = tid + 256 * u;
+      const int key = c / d8, off = (c % d8) * 8;
+      const int pg = key < 16 ? pg0 : pg1;
+      kr[u] = c < 32 * d8 ? ld16(kc + (((int64_t)pg * G + g) * 16 + (key & 15)) * D + off) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < NVC; ++u) {
+      const int c = tid + 256 * u;
+      const int col = c >> 2, half = (c >> 1) & 1, sub = c & 1;
+      const int pg = half ? pg1 : pg0;
+      vr[u] = col < V ? ld16(vt + (((int64_t)pg * G + g) * V + col) * 16 + 8 * sub) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < NKC; ++u) {
+      const int c = tid + 256 * u;
+      if (c < 32 * d8) *reinterpret_cast<uint4*>(&kl[buf][c / d8][(c % d8) * 8]) = kr[u];
+    }
+#pragma unroll
+    for (int u = 0; u < NVC; ++u) {
+      const int c = tid + 256 * u;
+      const int col = c >> 2;
+      if (col < V) *reinterpret_cast<uint4*>(&vl[buf][col][16 * ((c >> 1) & 1) + 8 * (c & 1)]) = vr[u];
+    }
+  };
+  __syncthreads();  // the zero fill is done before the first tile is staged
+  fetch(jt0);
+  int buf = 0;
+  // a buffer is rewritten two tiles later, after the barrier of the tile in between, which every wave
+  // reaches only when it has finished reading it
+  for (int jt = jt0; jt <= jt1; ++jt) {
+    stage(buf);
+    __syncthreads();
+    if (jt < jt1) fetch(jt + 1);
+    const int kbase = 32 * jt;
+    if (active && kbase + 31 >= klow && kbase <= pmaxw) {  // wave-uniform: some row of the wave may see the tile
+      f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < NQF; ++kk)
+        if (kk < nqf) {
+          s0 = mfma16(qf[kk], as_bf16x8(*reinterpret_cast<const uint4*>(&kl[buf][lr][32 * kk + 8 * lg])), s0);
+          s1 = mfma16(qf[kk], as_bf16x8(*reinterpret_cast<const uint4*>(&kl[buf][16 + lr][32 * kk + 8 * lg])), s1);
+        }
+      softmax_tile(s0, s1, kbase, false);
+      const bf16x8 pf = as_bf16x8(*reinterpret_cast<const uint4*>(&pl[wv][lr][8 * lg]));
+#pragma unroll
+      for (int ct = 0; ct < NCT; ++ct)
+        if (ct < nct)
+          O[ct] = mfma16(pf, as_bf16x8(*reinterpret_cast<const uint4*>(&vl[buf][16 * ct + lr][8 * lg])), O[ct]);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // P tile read before the next tile overwrites it
+    }
+    buf ^= 1;
+  }
+  if (!active) return;
+  const int vrot = a.v_freq != nullptr ? 2 * (V / 2) : 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float inv = 1.f / group16_sum(lsum[i]);
+    const int r = row0 + 4 * lg + i;
+    const bool ok = r < nrows;
+    const float fp = -(float)(pos0 + (ok ? r / rep : 0));
+    bf16_t* orow = out + ((int64_t)(t0 + (ok ? r / rep : 0)) * H + g * rep + (ok ? r % rep : 0)) * V;
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct) {
+      const int col = 16 * ct + lr;
+      float y = O[ct][i] * inv;
+      if (vrot > 0) {
+        const float other = __shfl_xor(y, 1, 64);
+        if (col < vrot) {
+          const float ang = fp * a.v_freq[col >> 1];
+          const float cs = cosf(ang), sn = sinf(ang);
+          y = (col & 1) ? (y * cs + other * sn) : (y * cs - other * sn);
+        }
+      }
+      if (ok && ct < nct && col < V) orow[col] = f2bf(y);
+    }
+  }
+}
+
 template <int NCT, int NQF>
 void launch_window_mfma(const WindowArgs& a, const void* q, float scale, const void* vt, int num_pages, void* out,
                         hipStream_t st) {
@@ -598,11 +823,16 @@ void launch_window_mfma(const WindowArgs& a, const void* q, float scale, const v
   const bf16_t* vp = reinterpret_cast<const bf16_t*>(vt);
   bf16_t* op = reinterpret_cast<bf16_t*>(out);
   const float sl = scale * 1.4426950408889634f;
-  // few rows per sequence (decoded tokens): few workgroups, so eight waves each stream the keys; else four
+  // few rows per sequence (decoded tokens): few workgroups, so eight waves each stream the keys of 16 rows;
+  // prompt portions: 64 rows per workgroup over key / value tiles staged in LDS (or, by a.prefill_kernel == 1,
+  // 16 rows per workgroup with the key tiles shared out over four waves)
   if ((int64_t)a.T * rep <= 16 * (int64_t)a.S)
     hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 8>), dim3(blocks, a.G), dim3(512), 0, st, a, qp, sl, vp, num_pages, op);
-  else
+  else if (a.prefill_kernel == 1 || NCT > 8)
     hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 4>), dim3(blocks, a.G), dim3(256), 0, st, a, qp, sl, vp, num_pages, op);
+  else
+    hipLaunchKernelGGL((window_attn_tiled_kernel<NCT, NQF>), dim3((a.T * rep + 63) / 64 + a.S, a.G), dim3(256), 0, st, a, qp, sl,
+                       vp, num_pages, op);
 }
 
 int heads_per_block(const WindowArgs& a) {

@@ -397,7 +397,8 @@ void window_pool(const Tensor& kc, const Tensor& vc, const OptT& kp, const OptT&
 
 void window_attn(const Tensor& q, const Tensor& kc, const Tensor& vc, const OptT& kp, const OptT& vp,
                  const Tensor& block_tables, const Tensor& context_lens, const Tensor& query_start, Tensor& out,
-                 double scale, int64_t H, int64_t window, int64_t pool, const OptT& sink, const OptT& v_freq, const OptT& vt) {
+                 double scale, int64_t H, int64_t window, int64_t pool, const OptT& sink, const OptT& v_freq, const OptT& vt,
+                 int64_t prefill_kernel) {
   auto a = window_common(kc, vc, kp, vp, H, pool);
   window_seq_meta(a, block_tables, query_start);
   a.context_lens = i32p(context_lens, "context_lens", a.S);
@@ -410,6 +411,8 @@ void window_attn(const Tensor& q, const Tensor& kc, const Tensor& vc, const OptT
   a.sink = f32p(sink, "sink", H);
   a.v_freq = f32p(v_freq, "v_freq", a.V / 2);
   const void* vtp = window_vt(vt, vc);
+  TORCH_CHECK(prefill_kernel == 0 || prefill_kernel == 1, "window_attn: prefill_kernel 0 or 1");
+  a.prefill_kernel = (int)prefill_kernel;
   c10::DeviceGuard guard(q.device());
   vgate::launch_window_attn(a, q.data_ptr(), (float)scale, out.data_ptr(), vtp, (int)kc.size(0), cur_stream());
 }
@@ -533,7 +536,7 @@ void bind_seq(pybind11::module& m) {
   m.def("window_attn", &window_attn, "sliding-window attention with pooled blocks and an optional sink", py::arg("q"),
         py::arg("kc"), py::arg("vc"), py::arg("kp"), py::arg("vp"), py::arg("block_tables"), py::arg("context_lens"),
         py::arg("query_start"), py::arg("out"), py::arg("scale"), py::arg("H"), py::arg("window"), py::arg("pool"),
-        py::arg("sink"), py::arg("v_freq"), py::arg("vt") = py::none());
+        py::arg("sink"), py::arg("v_freq"), py::arg("vt") = py::none(), py::arg("prefill_kernel") = 0);
   m.def("linear_attn_scratch", [](int64_t T, int64_t S, int64_t H, int64_t D, int64_t V) {
     return (int64_t)vgate::linear_attn_scratch_floats((int)T, (int)S, (int)H, (int)D, (int)V);
   }, "fp32 elements of scratch a linear_attn call over T rows and S sequences needs");

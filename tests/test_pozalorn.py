@@ -372,7 +372,7 @@ def _step_meta(lens_new, ctx, tables, d):
     return i32(pos), i32(slots), i32(qs), i32(ctx)
 
 
-def _run_window(d, dt, q, k, v, H, G, size, pool, sink, turn, tables, steps, transposed=False):
+def _run_window(d, dt, q, k, v, H, G, size, pool, sink, turn, tables, steps, transposed=False, prefill_kernel=0):
     """Feed sequences through window_write / window_pool / window_attn in the given steps
     (``steps``: list of per-sequence new-token counts); returns each sequence's outputs [T, H * V].
     ``transposed``: keep the transposed value copy, which selects the MFMA kernel (GPU, bf16)."""
@@ -403,7 +403,7 @@ def _run_window(d, dt, q, k, v, H, G, size, pool, sink, turn, tables, steps, tra
         if pool:
             seq.window_pool(kc, vc, kp, vp, pos, bt, qs, pool)
         o = torch.zeros(T, H * V, dtype=dt, device=d)
-        seq.window_attn(qo, kc, vc, kp, vp, bt, cl, qs, o, 0.5, H, size, pool, sink, vf, vt=vt)
+        seq.window_attn(qo, kc, vc, kp, vp, bt, cl, qs, o, 0.5, H, size, pool, sink, vf, vt=vt, prefill_kernel=prefill_kernel)
         for s in range(S):
             outs[s].append(o[int(qs[s]): int(qs[s + 1])].float().cpu())
         done = ctx
@@ -461,8 +461,10 @@ def test_window_attention_edges(device, f32, size, pool):
         want = _want_window(q, k, v, H, G, size, pool, sk, turn)
         skd = sk.to(d) if use_sink else None
         for steps in ([[T]], [[61], [2], [35], [1], [1], [50]], [[T - 40]] + [[1]] * 40):
-            for mfma in ([False, True] if device == "cuda" and not f32 else [False]):
-                got = _run_window(d, dt, [q], [k], [v], H, G, size, pool, skd, turn, tables, steps, transposed=mfma)[0]
+            # FMA kernel; on the GPU in bf16 also the two MFMA kernels for prompt portions (0: LDS-staged, 1: split)
+            for mfma in ([None, 0, 1] if device == "cuda" and not f32 else [None]):
+                got = _run_window(d, dt, [q], [k], [v], H, G, size, pool, skd, turn, tables, steps, transposed=mfma is not None,
+                                  prefill_kernel=mfma or 0)[0]
                 assert rel(got, want) < (3e-5 if f32 else 2e-2), (use_sink, turn, len(steps), mfma)
         # the crafted keys matter: one more or one fewer key in the window moves the answer
         # (with pool 1 every earlier token is seen either way, as itself or as its own block)
@@ -488,9 +490,10 @@ def test_window_attention_batch_and_page_reuse(device):
     got = _run_window(d, torch.float32, [qb], [kb], [vb], H, G, 10, 4, None, True, [[3, 1, 4]], [[20], [17]])
     assert rel(got[0], wb) < 3e-5
     if device == "cuda":   # the MFMA kernel: rows of two sequences, of several tokens and of one
-        got = _run_window(d, torch.bfloat16, [qa, qb], [ka, kb], [va, vb], H, G, 10, 4, None, True,
-                          [[3, 1, 4, 0, 2], [6, 5, 7]], [[30, 1], [2, 30], [38, 6]], transposed=True)
-        assert rel(got[0], wa) < 2e-2 and rel(got[1], wb) < 2e-2
+        for kern in (0, 1):
+            got = _run_window(d, torch.bfloat16, [qa, qb], [ka, kb], [va, vb], H, G, 10, 4, None, True,
+                              [[3, 1, 4, 0, 2], [6, 5, 7]], [[30, 1], [2, 30], [38, 6]], transposed=True, prefill_kernel=kern)
+            assert rel(got[0], wa) < 2e-2 and rel(got[1], wb) < 2e-2, kern
 
 
 @pytest.mark.parametrize("device", DEVICES)

@@ -417,15 +417,17 @@ def window_pool(kc, vc, kp, vp, positions, block_tables, query_start, pool: int,
 
 
 def window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out, scale: float, H: int, window: int,
-                pool: int, sink, v_freq, num_seqs: int | None = None, vt=None) -> None:
+                pool: int, sink, v_freq, num_seqs: int | None = None, vt=None, prefill_kernel: int = 0) -> None:
     """out[t, h] = sum_j p_j value_j over the keys position i of token t sees: the tokens j with
     0 <= i - j < window and, with ``pool`` = P > 0, the pooled row of every block b with
     b P + P - 1 <= i - window; p = softmax(scale q . key) over both kinds together, with exp(sink[h]) added
     to the denominator if ``sink`` is given. With ``v_freq`` the result is turned back by -i over all of V.
     Query head h reads key/value head h / (H / G). With ``vt`` (see :func:`window_write`) bf16 caches run
-    the MFMA kernel."""
+    the MFMA kernels (``prefill_kernel``: which one prompt portions take, 0 = tiles staged in LDS for 64 rows,
+    1 = 16 rows per workgroup with the tiles shared out over its waves)."""
     if q.is_cuda:
-        _C().window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out, scale, H, window, pool, sink, v_freq, vt)
+        _C().window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out, scale, H, window, pool, sink, v_freq, vt,
+                         prefill_kernel)
         return
     G, page, D, V = kc.shape[1], kc.shape[2], kc.shape[3], vc.shape[3]
     rep = H // G
